@@ -1,0 +1,129 @@
+// Decoupled-weight-decay Adam step on one flat parameter chunk, gfx950.
+//
+// Update order and fp32 arithmetic follow the reference Triton kernel
+// (flextrain/ops/_kernels/adamw.py:34-60):
+//   p -= (lr*wd)*p;  m = b1*m + (1-b1)*g;  v = b2*v + (1-b2)*g*g;
+//   p -= lr * ((m/bc1) / (sqrt(v/bc2) + eps))
+// with bc1/bc2 = 1 - beta^step computed by the host in double and passed as
+// fp32.  p, m, v are updated in place in whatever dtype each buffer has.
+// An optional extra output receives the updated parameter rounded to bf16 (the
+// compute-dtype copy a host-offloaded fp32 master needs); it has no
+// counterpart in the reference kernel.
+#include "common.h"
+#include "flexhip.h"
+
+namespace fx {
+
+constexpr int ADAM_THREADS = 256;
+
+struct AdamScalars {
+    float lr_wd, lr, beta1, omb1, beta2, omb2, eps, bc1, bc2;
+};
+
+FX_DEV void adam_elem(float& p, float g, float& m, float& v, const AdamScalars& a) {
+    p = p - a.lr_wd * p;
+    m = a.beta1 * m + a.omb1 * g;
+    v = a.beta2 * v + a.omb2 * (g * g);
+    const float mh = m / a.bc1;
+    const float vh = v / a.bc2;
+    const float denom = sqrtf(vh) + a.eps;
+    p = p - a.lr * (mh / denom);
+}
+
+template <typename TP, typename TG, typename TS, bool COPY>
+__global__ __launch_bounds__(ADAM_THREADS) void adamw_kernel(
+    TP* __restrict__ P, const TG* __restrict__ G, TS* __restrict__ M, TS* __restrict__ V,
+    bf16* __restrict__ PCOPY, int64_t n, AdamScalars a) {
+    const int64_t off = ((int64_t)blockIdx.x * ADAM_THREADS + threadIdx.x) * 8;
+    if (off + 8 <= n) {
+        float p[8], g[8], m[8], v[8];
+        load_f32<TP, 8>(P + off, p);
+        load_f32<TG, 8>(G + off, g);
+        load_f32<TS, 8>(M + off, m);
+        load_f32<TS, 8>(V + off, v);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) adam_elem(p[j], g[j], m[j], v[j], a);
+        store_f32<TP, 8>(P + off, p);
+        store_f32<TS, 8>(M + off, m);
+        store_f32<TS, 8>(V + off, v);
+        if (COPY) store_f32<bf16, 8>(PCOPY + off, p);
+    } else {
+        for (int64_t i = off; i < n; ++i) {
+            float p = (float)P[i], g = (float)G[i], m = (float)M[i], v = (float)V[i];
+            adam_elem(p, g, m, v, a);
+            P[i] = (TP)p;
+            M[i] = (TS)m;
+            V[i] = (TS)v;
+            if (COPY) PCOPY[i] = (bf16)p;
+        }
+    }
+}
+
+// flag[0] |= 1 if any element is NaN or +-Inf.
+template <typename T>
+__global__ __launch_bounds__(256) void nonfinite_kernel(const T* __restrict__ X, int64_t n,
+                                                        int* __restrict__ flag) {
+    int bad = 0;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+        const float v = (float)X[i];
+        bad |= !(fabsf(v) <= 3.402823466e38f);
+    }
+    if (__any(bad) && (threadIdx.x & 63) == 0) atomicOr(flag, 1);
+}
+
+template <typename TP, typename TG, typename TS>
+static void launch_adamw(void* p, const void* g, void* m, void* v, void* pcopy, int64_t n,
+                         const AdamScalars& a, hipStream_t s) {
+    const unsigned grid = (unsigned)((n + (int64_t)ADAM_THREADS * 8 - 1) / ((int64_t)ADAM_THREADS * 8));
+    if (pcopy)
+        adamw_kernel<TP, TG, TS, true><<<grid, ADAM_THREADS, 0, s>>>(
+            reinterpret_cast<TP*>(p), reinterpret_cast<const TG*>(g), reinterpret_cast<TS*>(m),
+            reinterpret_cast<TS*>(v), reinterpret_cast<bf16*>(pcopy), n, a);
+    else
+        adamw_kernel<TP, TG, TS, false><<<grid, ADAM_THREADS, 0, s>>>(
+            reinterpret_cast<TP*>(p), reinterpret_cast<const TG*>(g), reinterpret_cast<TS*>(m),
+            reinterpret_cast<TS*>(v), nullptr, n, a);
+}
+
+}  // namespace fx
+
+using namespace fx;
+
+extern "C" int fx_adamw_step(void* p, const void* g, void* m, void* v, void* p_bf16_out, int64_t n,
+                             int p_dt, int g_dt, int state_dt, float lr, float beta1, float beta2,
+                             float eps, float weight_decay, float bias_correction1,
+                             float bias_correction2, hipStream_t stream) {
+    if (n < 0) FX_FAIL("fx_adamw_step: negative element count");
+    if (n == 0) return 0;
+    if (!p || !g || !m || !v) FX_FAIL("fx_adamw_step: null pointer");
+    if (!aligned16(p) || !aligned16(g) || !aligned16(m) || !aligned16(v) ||
+        (p_bf16_out && !aligned16(p_bf16_out)))
+        FX_FAIL("fx_adamw_step: buffers must be 16-byte aligned");
+    AdamScalars a;
+    a.lr_wd = lr * weight_decay;
+    a.lr = lr;
+    a.beta1 = beta1;
+    a.omb1 = 1.0f - beta1;
+    a.beta2 = beta2;
+    a.omb2 = 1.0f - beta2;
+    a.eps = eps;
+    a.bc1 = bias_correction1;
+    a.bc2 = bias_correction2;
+    FX_DISPATCH_DTYPE(p_dt, TP,
+        FX_DISPATCH_DTYPE(g_dt, TG,
+            FX_DISPATCH_DTYPE(state_dt, TS,
+                launch_adamw<TP, TG, TS>(p, g, m, v, p_bf16_out, n, a, stream))));
+    FX_CHECK_LAUNCH("fx_adamw_step");
+    return 0;
+}
+
+extern "C" int fx_nonfinite_flag(const void* x, int64_t n, int dt, int* flag, hipStream_t stream) {
+    if (n < 0 || !flag) FX_FAIL("fx_nonfinite_flag: bad arguments");
+    if (n == 0) return 0;
+    int64_t blocks = (n + 255) / 256;
+    if (blocks > 2048) blocks = 2048;
+    FX_DISPATCH_DTYPE(dt, T,
+        nonfinite_kernel<T><<<(unsigned)blocks, 256, 0, stream>>>(reinterpret_cast<const T*>(x), n, flag));
+    FX_CHECK_LAUNCH("fx_nonfinite_flag");
+    return 0;
+}

@@ -1,0 +1,130 @@
+// Shared device helpers for the gfx950 (CDNA4, wave64) kernels.
+//
+// Element types are the three the C ABI's dtype enum names (0 = fp32, 1 = fp16,
+// 2 = bf16; same numbering as the reference GEMM dispatcher,
+// helpers/matmul_dispatcher/src/dispatch.cpp:19-21).  All math is done in fp32;
+// the helpers here move 16 bytes per lane per access.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+#include <stdio.h>
+
+namespace fx {
+
+typedef __bf16 bf16;
+typedef _Float16 f16;
+
+enum : int { DT_F32 = 0, DT_F16 = 1, DT_BF16 = 2 };
+
+constexpr int WAVE = 64;
+
+#define FX_DEV __device__ __forceinline__
+
+// ---------------------------------------------------------------------------
+// 16-byte vector packs: VecOf<T>::N elements of T in one global_load_dwordx4.
+// ---------------------------------------------------------------------------
+template <typename T> struct VecOf;
+template <> struct VecOf<float> { static constexpr int N = 4; typedef float type __attribute__((ext_vector_type(4))); };
+template <> struct VecOf<bf16>  { static constexpr int N = 8; typedef bf16  type __attribute__((ext_vector_type(8))); };
+template <> struct VecOf<f16>   { static constexpr int N = 8; typedef f16   type __attribute__((ext_vector_type(8))); };
+
+template <typename T> FX_DEV float to_f32(T v) { return (float)v; }
+template <typename T> FX_DEV T from_f32(float v) { return (T)v; }
+
+// Load/store `N` consecutive elements (N * sizeof(T) must be 16 or 32 bytes and
+// the address 16-byte aligned) converting to/from fp32 registers.
+template <typename T, int N>
+FX_DEV void load_f32(const T* __restrict__ p, float (&out)[N]) {
+    constexpr int VN = VecOf<T>::N;
+    static_assert(N % VN == 0, "N must be a multiple of the 16-byte pack");
+    typedef typename VecOf<T>::type V;
+#pragma unroll
+    for (int i = 0; i < N / VN; ++i) {
+        V v = *reinterpret_cast<const V*>(p + i * VN);
+#pragma unroll
+        for (int j = 0; j < VN; ++j) out[i * VN + j] = (float)v[j];
+    }
+}
+
+template <typename T, int N>
+FX_DEV void store_f32(T* __restrict__ p, const float (&in)[N]) {
+    constexpr int VN = VecOf<T>::N;
+    static_assert(N % VN == 0, "N must be a multiple of the 16-byte pack");
+    typedef typename VecOf<T>::type V;
+#pragma unroll
+    for (int i = 0; i < N / VN; ++i) {
+        V v;
+#pragma unroll
+        for (int j = 0; j < VN; ++j) v[j] = (T)in[i * VN + j];
+        *reinterpret_cast<V*>(p + i * VN) = v;
+    }
+}
+
+// Round an fp32 value to T and back (the reference kernels round at a few
+// named points; this reproduces one such rounding).
+template <typename T> FX_DEV float round_to(float v) { return (float)(T)v; }
+
+// ---------------------------------------------------------------------------
+// Reductions.  `W` lanes (power of two, <= 64) that are contiguous in the wave
+// cooperate; every lane of the group ends with the group's sum.
+// ---------------------------------------------------------------------------
+template <int W>
+FX_DEV float group_sum(float v) {
+#pragma unroll
+    for (int off = W / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+template <int W>
+FX_DEV float group_max(float v) {
+#pragma unroll
+    for (int off = W / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+// Sum across `NWAVES` waves of a workgroup through LDS (smem needs NWAVES
+// floats).  All threads of the participating waves must call it.
+template <int NWAVES>
+FX_DEV float block_sum(float v, float* smem, int wave_in_group, int lane) {
+    v = group_sum<64>(v);
+    if (NWAVES == 1) return v;
+    __syncthreads();
+    if (lane == 0) smem[wave_in_group] = v;
+    __syncthreads();
+    float t = 0.f;
+#pragma unroll
+    for (int i = 0; i < NWAVES; ++i) t += smem[i];
+    return t;
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+inline int elem_size(int dt) { return dt == DT_F32 ? 4 : 2; }
+
+#define FX_CHECK_LAUNCH(name)                                                        \
+    do {                                                                             \
+        hipError_t e__ = hipGetLastError();                                          \
+        if (e__ != hipSuccess) {                                                     \
+            fprintf(stderr, "flexhip: %s launch failed: %s\n", name,                 \
+                    hipGetErrorString(e__));                                         \
+            return -1;                                                               \
+        }                                                                            \
+    } while (0)
+
+#define FX_FAIL(...)                                                                 \
+    do {                                                                             \
+        fprintf(stderr, "flexhip: " __VA_ARGS__);                                    \
+        fprintf(stderr, "\n");                                                       \
+        return -1;                                                                   \
+    } while (0)
+
+// Dispatch a callable templated on element type from a runtime dtype enum.
+#define FX_DISPATCH_DTYPE(dt, T, ...)                                                \
+    switch (dt) {                                                                    \
+        case fx::DT_F32:  { typedef float T;    __VA_ARGS__; break; }                \
+        case fx::DT_F16:  { typedef fx::f16 T;  __VA_ARGS__; break; }                \
+        case fx::DT_BF16: { typedef fx::bf16 T; __VA_ARGS__; break; }                \
+        default: FX_FAIL("unsupported dtype enum %d", (int)(dt));                    \
+    }
+
+}  // namespace fx

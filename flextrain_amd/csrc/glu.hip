@@ -1,0 +1,214 @@
+// Gated activations (SwiGLU, gated GELU-tanh), forward and backward, gfx950.
+//
+// out = act(x1) * x3, x1 = gate, x3 = up/value.  Math follows the reference
+// Triton kernels: flextrain/ops/_kernels/swiglu.py:9-96 and
+// flextrain/ops/_kernels/gelu_tanh_gated.py:55-140.  Pure streaming kernels:
+// every lane moves 16 bytes per tensor per access, two packs per lane.
+#include "common.h"
+#include "flexhip.h"
+
+namespace fx {
+
+enum : int { ACT_SILU = 0, ACT_GELU_TANH = 1 };
+
+FX_DEV float fast_sigmoid(float x) {
+    // 1 / (1 + 2^(-x*log2 e)); v_exp_f32 + v_rcp_f32, ~1 ulp each.
+    return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x));
+}
+
+template <typename T, int ACT>
+FX_DEV float glu_fwd_elem(float x1, float x3) {
+    if (ACT == ACT_SILU) {
+        const float s = fast_sigmoid(x1);
+        return (x1 * s) * x3;
+    } else {
+        const float cu = x1 * x1 * x1;
+        const float u = 0.7978845608028654f * (x1 + 0.044715f * cu);
+        const float th = 2.0f * fast_sigmoid(2.0f * u) - 1.0f;
+        const float g = 0.5f * x1 * (1.0f + th);
+        return g * x3;
+    }
+}
+
+template <typename T, int ACT>
+FX_DEV void glu_bwd_elem(float x1, float x3, float dout, float& dx1, float& dx3, float& act) {
+    if (ACT == ACT_SILU) {
+        const float s = fast_sigmoid(x1);
+        const float a = x1 * s;
+        act = a * x3;
+        dx3 = dout * a;
+        const float ds = s * (1.0f + x1 * (1.0f - s));
+        // The reference multiplies dout*x3 in the storage dtype before the fp32
+        // factor (swiglu.py:92); reproduce that one rounding.
+        dx1 = round_to<T>(dout * x3) * ds;
+    } else {
+        const float sq = x1 * x1;
+        const float cu = sq * x1;
+        const float u = 0.7978845608028654f * (x1 + 0.044715f * cu);
+        const float th = 2.0f * fast_sigmoid(2.0f * u) - 1.0f;
+        const float opt = 1.0f + th;
+        const float g = 0.5f * x1 * opt;
+        act = g * x3;
+        dx3 = dout * g;
+        const float du = 0.7978845608028654f * (1.0f + 3.0f * 0.044715f * sq);
+        const float sech = 1.0f - th * th;
+        const float dg = 0.5f * opt + 0.5f * x1 * sech * du;
+        dx1 = dout * x3 * dg;
+    }
+}
+
+constexpr int GLU_THREADS = 256;
+constexpr int GLU_UNROLL = 2;  // packs of 8 per lane
+
+template <typename T, typename TO, int ACT>
+__global__ __launch_bounds__(GLU_THREADS) void glu_fwd_kernel(
+    const T* __restrict__ X1, const T* __restrict__ X3, TO* __restrict__ OUT, int64_t n) {
+    const int64_t base = ((int64_t)blockIdx.x * GLU_UNROLL) * GLU_THREADS * 8;
+    float a[GLU_UNROLL][8], b[GLU_UNROLL][8];
+    bool full[GLU_UNROLL];
+#pragma unroll
+    for (int u = 0; u < GLU_UNROLL; ++u) {
+        const int64_t off = base + ((int64_t)u * GLU_THREADS + threadIdx.x) * 8;
+        full[u] = off + 8 <= n;
+        if (full[u]) {
+            load_f32<T, 8>(X1 + off, a[u]);
+            load_f32<T, 8>(X3 + off, b[u]);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < GLU_UNROLL; ++u) {
+        const int64_t off = base + ((int64_t)u * GLU_THREADS + threadIdx.x) * 8;
+        if (full[u]) {
+            float o[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) o[j] = glu_fwd_elem<T, ACT>(a[u][j], b[u][j]);
+            store_f32<TO, 8>(OUT + off, o);
+        } else {
+            for (int64_t i = off; i < n && i < off + 8; ++i)
+                OUT[i] = (TO)glu_fwd_elem<T, ACT>((float)X1[i], (float)X3[i]);
+        }
+    }
+}
+
+template <typename T, int ACT, bool STORE_ACT>
+__global__ __launch_bounds__(GLU_THREADS) void glu_bwd_kernel(
+    const T* __restrict__ X1, const T* __restrict__ X3, const T* __restrict__ DOUT,
+    T* __restrict__ DX1, T* __restrict__ DX3, T* __restrict__ ACTOUT, int64_t n) {
+    const int64_t base = ((int64_t)blockIdx.x * GLU_UNROLL) * GLU_THREADS * 8;
+    float a[GLU_UNROLL][8], b[GLU_UNROLL][8], d[GLU_UNROLL][8];
+    bool full[GLU_UNROLL];
+#pragma unroll
+    for (int u = 0; u < GLU_UNROLL; ++u) {
+        const int64_t off = base + ((int64_t)u * GLU_THREADS + threadIdx.x) * 8;
+        full[u] = off + 8 <= n;
+        if (full[u]) {
+            load_f32<T, 8>(X1 + off, a[u]);
+            load_f32<T, 8>(X3 + off, b[u]);
+            load_f32<T, 8>(DOUT + off, d[u]);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < GLU_UNROLL; ++u) {
+        const int64_t off = base + ((int64_t)u * GLU_THREADS + threadIdx.x) * 8;
+        if (full[u]) {
+            float g1[8], g3[8], ac[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                glu_bwd_elem<T, ACT>(a[u][j], b[u][j], d[u][j], g1[j], g3[j], ac[j]);
+            store_f32<T, 8>(DX1 + off, g1);
+            store_f32<T, 8>(DX3 + off, g3);
+            if (STORE_ACT) store_f32<T, 8>(ACTOUT + off, ac);
+        } else {
+            for (int64_t i = off; i < n && i < off + 8; ++i) {
+                float g1, g3, ac;
+                glu_bwd_elem<T, ACT>((float)X1[i], (float)X3[i], (float)DOUT[i], g1, g3, ac);
+                DX1[i] = (T)g1;
+                DX3[i] = (T)g3;
+                if (STORE_ACT) ACTOUT[i] = (T)ac;
+            }
+        }
+    }
+}
+
+// Unaligned-pointer fallback: one element per lane.
+template <typename T, typename TO, int ACT>
+__global__ __launch_bounds__(256) void glu_fwd_scalar_kernel(const T* X1, const T* X3, TO* OUT, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) OUT[i] = (TO)glu_fwd_elem<T, ACT>((float)X1[i], (float)X3[i]);
+}
+template <typename T, int ACT>
+__global__ __launch_bounds__(256) void glu_bwd_scalar_kernel(const T* X1, const T* X3, const T* DOUT,
+                                                             T* DX1, T* DX3, T* ACTOUT, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) {
+        float g1, g3, ac;
+        glu_bwd_elem<T, ACT>((float)X1[i], (float)X3[i], (float)DOUT[i], g1, g3, ac);
+        DX1[i] = (T)g1;
+        DX3[i] = (T)g3;
+        if (ACTOUT) ACTOUT[i] = (T)ac;
+    }
+}
+
+template <typename T, typename TO, int ACT>
+static void launch_glu_fwd(const void* x1, const void* x3, void* out, int64_t n, hipStream_t s) {
+    const T* a = reinterpret_cast<const T*>(x1);
+    const T* b = reinterpret_cast<const T*>(x3);
+    TO* o = reinterpret_cast<TO*>(out);
+    if (aligned16(x1) && aligned16(x3) && aligned16(out)) {
+        const int64_t per_block = (int64_t)GLU_UNROLL * GLU_THREADS * 8;
+        glu_fwd_kernel<T, TO, ACT><<<(unsigned)((n + per_block - 1) / per_block), GLU_THREADS, 0, s>>>(a, b, o, n);
+    } else {
+        glu_fwd_scalar_kernel<T, TO, ACT><<<(unsigned)((n + 255) / 256), 256, 0, s>>>(a, b, o, n);
+    }
+}
+
+template <typename T, int ACT>
+static void launch_glu_bwd(const void* x1, const void* x3, const void* dout, void* dx1, void* dx3,
+                           void* act, int64_t n, hipStream_t s) {
+    const T* a = reinterpret_cast<const T*>(x1);
+    const T* b = reinterpret_cast<const T*>(x3);
+    const T* d = reinterpret_cast<const T*>(dout);
+    T* g1 = reinterpret_cast<T*>(dx1);
+    T* g3 = reinterpret_cast<T*>(dx3);
+    T* ac = reinterpret_cast<T*>(act);
+    if (aligned16(x1) && aligned16(x3) && aligned16(dout) && aligned16(dx1) && aligned16(dx3) &&
+        (act == nullptr || aligned16(act))) {
+        const int64_t per_block = (int64_t)GLU_UNROLL * GLU_THREADS * 8;
+        const unsigned grid = (unsigned)((n + per_block - 1) / per_block);
+        if (act) glu_bwd_kernel<T, ACT, true><<<grid, GLU_THREADS, 0, s>>>(a, b, d, g1, g3, ac, n);
+        else glu_bwd_kernel<T, ACT, false><<<grid, GLU_THREADS, 0, s>>>(a, b, d, g1, g3, ac, n);
+    } else {
+        glu_bwd_scalar_kernel<T, ACT><<<(unsigned)((n + 255) / 256), 256, 0, s>>>(a, b, d, g1, g3, ac, n);
+    }
+}
+
+}  // namespace fx
+
+using namespace fx;
+
+extern "C" int fx_glu_fwd(const void* x1, const void* x3, void* out, int64_t n, int in_dt,
+                          int out_dt, int act, hipStream_t stream) {
+    if (n < 0) FX_FAIL("fx_glu_fwd: negative element count");
+    if (n == 0) return 0;
+    if (!x1 || !x3 || !out) FX_FAIL("fx_glu_fwd: null pointer");
+    if (act != ACT_SILU && act != ACT_GELU_TANH) FX_FAIL("fx_glu_fwd: unknown activation %d", act);
+    FX_DISPATCH_DTYPE(in_dt, T,
+        FX_DISPATCH_DTYPE(out_dt, TO,
+            if (act == ACT_SILU) launch_glu_fwd<T, TO, ACT_SILU>(x1, x3, out, n, stream);
+            else launch_glu_fwd<T, TO, ACT_GELU_TANH>(x1, x3, out, n, stream)));
+    FX_CHECK_LAUNCH("fx_glu_fwd");
+    return 0;
+}
+
+extern "C" int fx_glu_bwd(const void* x1, const void* x3, const void* dout, void* dx1, void* dx3,
+                          void* act_out, int64_t n, int dt, int act, hipStream_t stream) {
+    if (n < 0) FX_FAIL("fx_glu_bwd: negative element count");
+    if (n == 0) return 0;
+    if (!x1 || !x3 || !dout || !dx1 || !dx3) FX_FAIL("fx_glu_bwd: null pointer");
+    if (act != ACT_SILU && act != ACT_GELU_TANH) FX_FAIL("fx_glu_bwd: unknown activation %d", act);
+    FX_DISPATCH_DTYPE(dt, T,
+        if (act == ACT_SILU) launch_glu_bwd<T, ACT_SILU>(x1, x3, dout, dx1, dx3, act_out, n, stream);
+        else launch_glu_bwd<T, ACT_GELU_TANH>(x1, x3, dout, dx1, dx3, act_out, n, stream));
+    FX_CHECK_LAUNCH("fx_glu_bwd");
+    return 0;
+}

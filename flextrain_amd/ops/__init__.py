@@ -1,0 +1,39 @@
+"""The ``flextrain_*`` op surface (flextrain/ops/__init__.py:14-120) for the
+ops on the per-layer training compute path, backed by libflexhip.so."""
+from __future__ import annotations
+
+from .adamw import flextrain_adamw_step
+from .glu import (
+    flextrain_gelu_tanh_gated_bwd,
+    flextrain_gelu_tanh_gated_fwd,
+    flextrain_swiglu_bwd,
+    flextrain_swiglu_fwd,
+)
+from .rmsnorm import (
+    flextrain_rmsnorm_bwd,
+    flextrain_rmsnorm_fwd,
+    flextrain_rmsnorm_fwd_recompute,
+)
+from .rope import (
+    build_rope_inv_freq,
+    flextrain_rope_bwd,
+    flextrain_rope_fwd,
+    flextrain_rope_partial_bwd,
+    flextrain_rope_partial_fwd,
+)
+
+__all__ = [
+    "build_rope_inv_freq",
+    "flextrain_adamw_step",
+    "flextrain_gelu_tanh_gated_bwd",
+    "flextrain_gelu_tanh_gated_fwd",
+    "flextrain_rmsnorm_bwd",
+    "flextrain_rmsnorm_fwd",
+    "flextrain_rmsnorm_fwd_recompute",
+    "flextrain_rope_bwd",
+    "flextrain_rope_fwd",
+    "flextrain_rope_partial_bwd",
+    "flextrain_rope_partial_fwd",
+    "flextrain_swiglu_bwd",
+    "flextrain_swiglu_fwd",
+]

@@ -1,0 +1,119 @@
+/* flexhip: C ABI of the MI355X (gfx950) per-layer training compute path.
+ *
+ * One shared library, libflexhip.so, exports everything below.  Conventions,
+ * shared by every entry point unless its comment says otherwise:
+ *   - plain pointers and sizes only; device pointers are raw HIP addresses;
+ *   - the caller owns every buffer, including scratch ("ws") buffers whose
+ *     size the matching *_ws_bytes() function reports; the library never
+ *     allocates or frees device memory;
+ *   - work is enqueued on the given stream and the call returns without
+ *     synchronising;
+ *   - dtype enums: 0 = fp32, 1 = fp16, 2 = bf16
+ *     (numbering of helpers/matmul_dispatcher/src/dispatch.cpp:19-21);
+ *   - return 0 on success, -1 on failure with one line on stderr
+ *     (convention of helpers/matmul_dispatcher/src/dispatch.cpp:193-197).
+ *
+ * Each declaration cites the reference interface it stands in for; paths are
+ * relative to the root of als244/flextrain.
+ */
+#ifndef FLEXHIP_H
+#define FLEXHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#ifndef __HIP__
+typedef struct ihipStream_t* hipStream_t;
+#endif
+
+#define FX_DT_F32 0
+#define FX_DT_F16 1
+#define FX_DT_BF16 2
+
+#define FX_ACT_SILU 0
+#define FX_ACT_GELU_TANH 1
+
+/* Library identification: returns a static string "flexhip <version> gfx950". */
+const char* fx_version(void);
+
+/* ---- RMSNorm ----------------------------------------------------------- */
+
+/* flextrain_rmsnorm_fwd and flextrain_rmsnorm_fwd_recompute
+ * (flextrain/ops/_kernels/rmsnorm.py:456-530, :532-583; kernels :9-163).
+ * x, y: (rows, ncols) contiguous, same dtype x_dt; y may alias x.  w: (ncols,)
+ * of dtype w_dt or NULL.  rstd: fp32 (rows,), written when use_saved_rstd == 0
+ * and read when it is 1.  Per-head normalisation is the call with
+ * rows = T*H, ncols = head_dim. */
+int fx_rmsnorm_fwd(const void* x, const void* w, void* y, float* rstd, int64_t rows, int ncols,
+                   float eps, int x_dt, int w_dt, int use_saved_rstd, hipStream_t stream);
+
+/* Scratch bytes fx_rmsnorm_bwd needs for its dW partial sums (0 when the
+ * shape takes the unvectorised path).  Replaces the torch.empty partial buffer
+ * of flextrain/ops/_kernels/rmsnorm.py:786-789. */
+size_t fx_rmsnorm_bwd_ws_bytes(int64_t rows, int ncols);
+
+/* flextrain_rmsnorm_bwd (flextrain/ops/_kernels/rmsnorm.py:585-832; kernels
+ * :170-412).  dy, x, dx, y_out share dtype x_dt.  accumulate_dx: dx += result.
+ * dw (dtype dw_dt, (ncols,)) is written, or added to when accumulate_dw; pass
+ * dw = NULL or w = NULL to skip the weight gradient.  y_out != NULL
+ * re-materialises the forward output. */
+int fx_rmsnorm_bwd(const void* dy, const void* x, const void* w, const float* rstd, void* dx,
+                   int accumulate_dx, void* dw, int dw_dt, int accumulate_dw, void* y_out,
+                   int64_t rows, int ncols, int x_dt, int w_dt, float* ws, size_t ws_bytes,
+                   hipStream_t stream);
+
+/* ---- Rotary embedding -------------------------------------------------- */
+
+/* flextrain_rope_fwd / flextrain_rope_bwd (flextrain/ops/_kernels/rope.py:207-307;
+ * kernels :8-157) and, with rot_dim < D, flextrain_rope_partial_fwd/bwd
+ * (flextrain/ops/_kernels/rope_partial.py:29-147).  In place on q (T,Hq,D) and
+ * k (T,Hk,D); k may be NULL with Hk = 0.  Strides are in elements, three per
+ * tensor (token, head, channel).  pos: int32, element t at pos[t*stride_pos];
+ * inv_freq: fp32, pair i at inv_freq[i*stride_if], rot_dim/2 entries. */
+int fx_rope(void* q, void* k, const int32_t* pos, int64_t stride_pos, const float* inv_freq,
+            int64_t stride_if, int64_t T_tokens, int Hq, int Hk, int D, int rot_dim,
+            const int64_t* q_strides, const int64_t* k_strides, int dt, int backward,
+            hipStream_t stream);
+
+/* ---- Gated activations ------------------------------------------------- */
+
+/* flextrain_swiglu_fwd (flextrain/ops/_kernels/swiglu.py:103-133) for
+ * act = FX_ACT_SILU and flextrain_gelu_tanh_gated_fwd
+ * (flextrain/ops/_kernels/gelu_tanh_gated.py:148-170) for FX_ACT_GELU_TANH.
+ * out[i] = act(x1[i]) * x3[i] over n contiguous elements. */
+int fx_glu_fwd(const void* x1, const void* x3, void* out, int64_t n, int in_dt, int out_dt, int act,
+               hipStream_t stream);
+
+/* flextrain_swiglu_bwd (flextrain/ops/_kernels/swiglu.py:136-182) and
+ * flextrain_gelu_tanh_gated_bwd (flextrain/ops/_kernels/gelu_tanh_gated.py:173-214).
+ * act_out != NULL also stores the recomputed forward output. */
+int fx_glu_bwd(const void* x1, const void* x3, const void* dout, void* dx1, void* dx3, void* act_out,
+               int64_t n, int dt, int act, hipStream_t stream);
+
+/* ---- AdamW ------------------------------------------------------------- */
+
+/* flextrain_adamw_step (flextrain/ops/_kernels/adamw.py:62-102; kernel :5-60).
+ * p (p_dt), m and v (state_dt) are updated in place; g has dtype g_dt.
+ * bias_correction{1,2} = 1 - beta^max(1,step), computed by the caller in
+ * double.  p_bf16_out, when not NULL, additionally receives bf16(p_new); the
+ * reference has no such output (its engine re-casts during the copy back to
+ * the host, flextrain/engine/buffers.py:1144-1164). */
+int fx_adamw_step(void* p, const void* g, void* m, void* v, void* p_bf16_out, int64_t n, int p_dt,
+                  int g_dt, int state_dt, float lr, float beta1, float beta2, float eps,
+                  float weight_decay, float bias_correction1, float bias_correction2,
+                  hipStream_t stream);
+
+/* The check_error branch of flextrain_adamw_step
+ * (flextrain/ops/_kernels/adamw.py:80-83): ORs 1 into *flag (device int32,
+ * caller-zeroed) if any element of x is NaN or infinite. */
+int fx_nonfinite_flag(const void* x, int64_t n, int dt, int* flag, hipStream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* FLEXHIP_H */
