@@ -1,0 +1,279 @@
+#!/usr/bin/env python3
+"""Throughput of the per-layer training compute path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extra] [--no-cpu]
+
+A "step" is one pass of the Llama-3.1-8B-shaped RoPE + SwiGLU forward+backward
+workload (q [8192,32,128], k [8192,8,128], gate/up/dout [8192,14336], bf16,
+synthetic N(0,1)) with every input already resident in HBM.  ``value`` is the
+algorithmic HBM bytes of a step divided by its wall time on the GPU stream.
+Every kernel launch inside the timed region is bracketed by HIP events on the
+launch stream, which gives the per-kernel average durations behind
+``roofline`` (dominant kernel: SwiGLU backward) and ``ops``.
+
+After the timed region the other single-GPU configurations (RMSNorm, AdamW, ...)
+are measured the same way and reported under ``ops``; they do not enter
+``value``.  The CPU baseline times the CPU oracle of the same workload on a
+bounded token sample on the host cores.
+
+Prints exactly one JSON line on stdout.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0       # MI355X HBM3E, published
+BF16_PEAK_TFLOPS = 2500.0    # MI355X dense bf16 MFMA, published
+
+METRIC = "per-op HBM GB/s (% of 8 TB/s) + lm_head/MoE GEMM TFLOPS (% bf16 MFMA peak)"
+
+
+def _parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-extra", action="store_true", help="skip the non-headline configurations")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    return ap.parse_args()
+
+
+class Timed:
+    """Accumulates HIP-event durations per named kernel on one stream."""
+
+    def __init__(self, torch, stream):
+        self.torch, self.stream = torch, stream
+        self.pairs = {}
+
+    def __call__(self, name, fn):
+        a = self.torch.cuda.Event(enable_timing=True)
+        b = self.torch.cuda.Event(enable_timing=True)
+        a.record(self.stream)
+        fn()
+        b.record(self.stream)
+        self.pairs.setdefault(name, []).append((a, b))
+
+    def mean_ms(self, name):
+        ev = self.pairs[name]
+        return sum(a.elapsed_time(b) for a, b in ev) / len(ev)
+
+    def clear(self):
+        self.pairs = {}
+
+
+def _op_entry(name, work, unit, ms):
+    """work: algorithmic bytes (unit GB/s) or FLOPs (unit TFLOP/s) per launch."""
+    if unit == "GB/s":
+        ach, peak = work / (ms * 1e-3) / 1e9, HBM_PEAK_GBPS
+    else:
+        ach, peak = work / (ms * 1e-3) / 1e12, BF16_PEAK_TFLOPS
+    return {"op": name, "algorithmic": work, "ms": round(ms, 5), "achieved": round(ach, 2),
+            "unit": unit, "frac": round(ach / peak, 4)}
+
+
+def _time_launches(torch, stream, fns, warmup=5, reps=20):
+    """Mean milliseconds per launch; ``fns`` is a list of equivalent closures over
+    distinct buffer sets, called round-robin so small working sets cannot sit in
+    the 256 MB last-level cache between launches."""
+    with torch.cuda.stream(stream):
+        for i in range(warmup):
+            fns[i % len(fns)]()
+        a = torch.cuda.Event(enable_timing=True)
+        b = torch.cuda.Event(enable_timing=True)
+        a.record(stream)
+        for i in range(reps):
+            fns[i % len(fns)]()
+        b.record(stream)
+        torch.cuda.synchronize()
+    return a.elapsed_time(b) / reps
+
+
+def run_extra(torch, ops, dev, stream, rn):
+    rows = []
+    # ---- configs[0]: RMSNorm fwd+bwd, x [2048,4096] bf16; 24 buffer sets = 1.6 GB
+    T, D, NSETS = 2048, 4096, 24
+    w = rn(D, std=0.02, mean=1.0).to(dev)
+    sets = []
+    for _ in range(NSETS):
+        x = rn(T, D).to(dev)
+        sets.append(dict(x=x, dy=torch.randn_like(x), y=torch.empty_like(x), dx=torch.empty_like(x),
+                         rstd=torch.empty(T, 1, dtype=torch.float32, device=dev)))
+    dw = torch.zeros(D, dtype=torch.float32, device=dev)
+    fwd = [lambda s=s: ops.flextrain_rmsnorm_fwd(s["x"], w, output=s["y"], rstd=s["rstd"]) for s in sets]
+    ms = _time_launches(torch, stream, fwd, warmup=NSETS, reps=4 * NSETS)
+    rows.append(_op_entry("c1.rmsnorm_fwd", 2 * T * D * 2 + D * 2 + T * 4, "GB/s", ms))
+    bwd = [lambda s=s: ops.flextrain_rmsnorm_bwd(s["dy"], s["x"], w, s["rstd"], dX=s["dx"], dW=dw) for s in sets]
+    for s in sets:
+        s["dx"].zero_()
+    ms = _time_launches(torch, stream, bwd, warmup=NSETS, reps=4 * NSETS)
+    # dX given => accumulate: reads dy, x, dx_old, writes dx (4 row tensors)
+    rows.append(_op_entry("c1.rmsnorm_bwd(dX+=,dW+=)", 4 * T * D * 2 + D * 2 + T * 4 + 2 * D * 4, "GB/s", ms))
+    bwd_e = [lambda s=s: ops.flextrain_rmsnorm_bwd(s["dy"], s["x"], w, s["rstd"], dX=s["dx"], dW=dw,
+                                                   recompute_output=True, recomputed_output_tensor=s["y"])
+             for s in sets]
+    ms = _time_launches(torch, stream, bwd_e, warmup=NSETS, reps=4 * NSETS)
+    rows.append(_op_entry("c1.rmsnorm_bwd(dX+=,dW+=,y)", 5 * T * D * 2 + D * 2 + T * 4 + 2 * D * 4, "GB/s", ms))
+    del sets, fwd, bwd, bwd_e
+    torch.cuda.empty_cache()
+
+    # ---- configs[3] kernel: AdamW on one 218,112,000-parameter chunk resident in HBM
+    n = 218_112_000
+    p = (torch.randn(n, device=dev) * 0.02)
+    m = torch.zeros(n, device=dev)
+    v = torch.zeros(n, device=dev)
+    gr = (torch.randn(n, device=dev) * 1e-3).to(torch.bfloat16)
+    pb = torch.empty(n, dtype=torch.bfloat16, device=dev)
+    hp = dict(lr=3e-5, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1)
+    step = [0]
+
+    def adam(copy):
+        step[0] += 1
+        ops.flextrain_adamw_step(p, gr, m, v, step=step[0], params_bf16_out=pb if copy else None, **hp)
+
+    ms = _time_launches(torch, stream, [lambda: adam(True)], warmup=3, reps=10)
+    rows.append(_op_entry("c4.adamw(fp32 p/m/v, bf16 g, bf16 copy-out)", 28 * n, "GB/s", ms))
+    ms = _time_launches(torch, stream, [lambda: adam(False)], warmup=3, reps=10)
+    rows.append(_op_entry("c4.adamw(fp32 p/m/v, bf16 g)", 26 * n, "GB/s", ms))
+    del p, m, v, gr, pb
+    torch.cuda.empty_cache()
+    return rows
+
+
+def main():
+    args = _parse()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU only (got --gpus {args.gpus}); "
+              "this path has no multi-GPU leg.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from flextrain_amd import ops
+    from flextrain_amd._lib import lib
+
+    lib()  # fail loudly before any timing if the native library is missing
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    stream = torch.cuda.Stream(device=dev)
+    timed = Timed(torch, stream)
+
+    # ------------------------------------------------------------------ inputs
+    T, HQ, HK, HD, F = 8192, 32, 8, 128, 14336
+    g = torch.Generator().manual_seed(1001)
+
+    def rn(*shape, dtype=torch.bfloat16, std=1.0, mean=0.0):
+        return (torch.randn(*shape, generator=g, dtype=torch.float32) * std + mean).to(dtype)
+
+    q, k = rn(T, HQ, HD).to(dev), rn(T, HK, HD).to(dev)
+    pos = torch.arange(T, dtype=torch.int32).view(T, 1).to(dev)
+    inv_freq = ops.build_rope_inv_freq(HD, 500000.0).to(dev)
+    gate, up, dout = rn(T, F).to(dev), rn(T, F).to(dev), rn(T, F).to(dev)
+    out, dgate, dup = torch.empty_like(gate), torch.empty_like(gate), torch.empty_like(gate)
+
+    rope_bytes = 2 * T * (HQ + HK) * HD * 2          # read + write, q and k
+    n = T * F
+    swiglu_fwd_bytes, swiglu_bwd_bytes = 3 * n * 2, 5 * n * 2
+    step_bytes = 2 * rope_bytes + swiglu_fwd_bytes + swiglu_bwd_bytes
+
+    def step(rec):
+        rec("rope_fwd", lambda: ops.flextrain_rope_fwd([q, k], pos, inv_freq))
+        rec("swiglu_fwd", lambda: ops.flextrain_swiglu_fwd(gate, up, out=out))
+        rec("swiglu_bwd", lambda: ops.flextrain_swiglu_bwd(gate, up, dout, dx1=dgate, dx3=dup))
+        rec("rope_bwd", lambda: ops.flextrain_rope_bwd([q, k], pos, inv_freq))
+
+    untimed = lambda name, fn: fn()
+    with torch.cuda.stream(stream):
+        for _ in range(args.warmup):
+            step(untimed)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step(timed)
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+
+    ms_per_step = wall * 1e3 / args.steps
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+    work = {"rope_fwd": rope_bytes, "rope_bwd": rope_bytes, "swiglu_fwd": swiglu_fwd_bytes,
+            "swiglu_bwd": swiglu_bwd_bytes}
+    op_rows = [_op_entry(f"c2.{name}", work[name], "GB/s", timed.mean_ms(name)) for name in work]
+    dom_ms = timed.mean_ms("swiglu_bwd")
+    dom_gbps = swiglu_bwd_bytes / (dom_ms * 1e-3) / 1e9
+    roofline = {"kernel": "glu_bwd_kernel<bf16, silu>", "bound": "hbm", "achieved": round(dom_gbps, 1),
+                "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(dom_gbps / HBM_PEAK_GBPS, 4),
+                "traffic": None, "algorithmic_bytes": swiglu_bwd_bytes, "avg_ms": round(dom_ms, 5)}
+    del q, k, gate, up, dout, out, dgate, dup
+
+    # ------------------------------------------------- other configurations
+    if not args.no_extra:
+        op_rows += run_extra(torch, ops, dev, stream, rn)
+
+    # -------------------------------------------------------- CPU baseline
+    cpu = None
+    if not args.no_cpu:
+        from oracle import glu as o_glu
+        from oracle import rope as o_rope
+
+        cores = os.cpu_count() or 1
+        torch.set_num_threads(cores)
+        Ts = 1024  # bounded sample: the first 1024 of the 8192 tokens
+        gs = torch.Generator().manual_seed(1001)
+        cq = torch.randn(Ts, HQ, HD, generator=gs).to(torch.bfloat16)
+        ck = torch.randn(Ts, HK, HD, generator=gs).to(torch.bfloat16)
+        cg, cu, cd = (torch.randn(Ts, F, generator=gs).to(torch.bfloat16) for _ in range(3))
+        cpos = torch.arange(Ts, dtype=torch.int32).view(Ts, 1)
+        cinv = o_rope.vanilla_inv_freq(HD, 500000.0)
+
+        def cpu_step():
+            o_rope.rope(cq, cpos, cinv), o_rope.rope(ck, cpos, cinv)
+            o_glu.swiglu_fwd(cg, cu)
+            o_glu.swiglu_bwd(cg, cu, cd)
+            o_rope.rope(cq, cpos, cinv, backward=True), o_rope.rope(ck, cpos, cinv, backward=True)
+
+        cpu_step()
+        times = []
+        t_begin = time.perf_counter()
+        while len(times) < 3 or (time.perf_counter() - t_begin < 10.0 and len(times) < 50):
+            t1 = time.perf_counter()
+            cpu_step()
+            times.append(time.perf_counter() - t1)
+        times.sort()
+        med = times[len(times) // 2]
+        cpu = {"value": round(step_bytes * (Ts / T) / med / 1e9, 3), "unit": "GB/s",
+               "cores": torch.get_num_threads(), "kind": "port",
+               "sample": f"CPU oracle (PyTorch fp32 formulas) on the first {Ts} of {T} tokens of the same "
+                         f"workload, median of {len(times)} runs, {med * 1e3:.1f} ms each"}
+
+    result = {
+        "metric": METRIC,
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16 storage, fp32 arithmetic",
+        "data": "synthetic",
+        "config": {"workload": "configs[1]: Llama-3.1-8B-shaped RoPE (q [8192,32,128], k [8192,8,128], "
+                               "theta 5e5) + SwiGLU (gate/up/dout [8192,14336]) forward+backward",
+                   "algorithmic_bytes_per_step": step_bytes},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "ops": op_rows,
+    }
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -47,6 +47,26 @@ _SIGNATURES = {
                               c_int, c_int, c_float, c_float, c_float, c_float, c_float, c_float,
                               c_float, c_void_p]),
     "fx_nonfinite_flag": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p]),
+    "fx_topk_softmax": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_int,
+                                c_void_p]),
+    "fx_moe_sort_ws_bytes": (c_size_t, [c_int64, c_int]),
+    "fx_moe_sort": (c_int, [c_void_p, c_int, c_int64, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
+                            c_size_t, c_void_p]),
+    "fx_copy_i32": (c_int, [c_void_p, c_void_p, c_int, c_void_p]),
+    "fx_router_gate_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+                                   c_int64, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "fx_load_balance_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_float, c_int,
+                                    c_int, c_void_p]),
+    "fx_moe_scatter": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int64, c_int, c_int,
+                               c_int64, c_int, c_void_p]),
+    "fx_moe_scatter_weights": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int, c_void_p]),
+    "fx_moe_gather": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
+                              c_int64, c_int, c_int, c_int, c_void_p]),
+    "fx_swiglu_moe_fwd": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int64, c_int, c_int64,
+                                  c_int64, c_int, c_void_p]),
+    "fx_swiglu_moe_bwd": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                                  c_int64, c_int, c_int64, c_int64, c_int64, c_int64, c_int, c_int,
+                                  c_void_p]),
 }
 
 _lib = None

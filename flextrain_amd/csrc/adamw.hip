@@ -30,23 +30,23 @@ FX_DEV void adam_elem(float& p, float g, float& m, float& v, const AdamScalars& 
     p = p - a.lr * (mh / denom);
 }
 
-template <typename TP, typename TG, typename TS, bool COPY>
+template <typename TP, typename TG, typename TS, bool COPY, bool NT>
 __global__ __launch_bounds__(ADAM_THREADS) void adamw_kernel(
     TP* __restrict__ P, const TG* __restrict__ G, TS* __restrict__ M, TS* __restrict__ V,
     bf16* __restrict__ PCOPY, int64_t n, AdamScalars a) {
     const int64_t off = ((int64_t)blockIdx.x * ADAM_THREADS + threadIdx.x) * 8;
     if (off + 8 <= n) {
         float p[8], g[8], m[8], v[8];
-        load_f32<TP, 8>(P + off, p);
-        load_f32<TG, 8>(G + off, g);
-        load_f32<TS, 8>(M + off, m);
-        load_f32<TS, 8>(V + off, v);
+        load_f32<TP, 8, NT>(P + off, p);
+        load_f32<TG, 8, NT>(G + off, g);
+        load_f32<TS, 8, NT>(M + off, m);
+        load_f32<TS, 8, NT>(V + off, v);
 #pragma unroll
         for (int j = 0; j < 8; ++j) adam_elem(p[j], g[j], m[j], v[j], a);
-        store_f32<TP, 8>(P + off, p);
-        store_f32<TS, 8>(M + off, m);
-        store_f32<TS, 8>(V + off, v);
-        if (COPY) store_f32<bf16, 8>(PCOPY + off, p);
+        store_f32<TP, 8, NT>(P + off, p);
+        store_f32<TS, 8, NT>(M + off, m);
+        store_f32<TS, 8, NT>(V + off, v);
+        if (COPY) store_f32<bf16, 8, NT>(PCOPY + off, p);
     } else {
         for (int64_t i = off; i < n; ++i) {
             float p = (float)P[i], g = (float)G[i], m = (float)M[i], v = (float)V[i];
@@ -75,14 +75,16 @@ template <typename TP, typename TG, typename TS>
 static void launch_adamw(void* p, const void* g, void* m, void* v, void* pcopy, int64_t n,
                          const AdamScalars& a, hipStream_t s) {
     const unsigned grid = (unsigned)((n + (int64_t)ADAM_THREADS * 8 - 1) / ((int64_t)ADAM_THREADS * 8));
-    if (pcopy)
-        adamw_kernel<TP, TG, TS, true><<<grid, ADAM_THREADS, 0, s>>>(
-            reinterpret_cast<TP*>(p), reinterpret_cast<const TG*>(g), reinterpret_cast<TS*>(m),
-            reinterpret_cast<TS*>(v), reinterpret_cast<bf16*>(pcopy), n, a);
-    else
-        adamw_kernel<TP, TG, TS, false><<<grid, ADAM_THREADS, 0, s>>>(
-            reinterpret_cast<TP*>(p), reinterpret_cast<const TG*>(g), reinterpret_cast<TS*>(m),
-            reinterpret_cast<TS*>(v), nullptr, n, a);
+    TP* P = reinterpret_cast<TP*>(p);
+    const TG* G = reinterpret_cast<const TG*>(g);
+    TS* M = reinterpret_cast<TS*>(m);
+    TS* V = reinterpret_cast<TS*>(v);
+    bf16* C = reinterpret_cast<bf16*>(pcopy);
+    const bool nt = (size_t)n * (2 * sizeof(TP) + sizeof(TG) + 4 * sizeof(TS)) >= kStreamingBytes;
+    if (pcopy && nt) adamw_kernel<TP, TG, TS, true, true><<<grid, ADAM_THREADS, 0, s>>>(P, G, M, V, C, n, a);
+    else if (pcopy) adamw_kernel<TP, TG, TS, true, false><<<grid, ADAM_THREADS, 0, s>>>(P, G, M, V, C, n, a);
+    else if (nt) adamw_kernel<TP, TG, TS, false, true><<<grid, ADAM_THREADS, 0, s>>>(P, G, M, V, C, n, a);
+    else adamw_kernel<TP, TG, TS, false, false><<<grid, ADAM_THREADS, 0, s>>>(P, G, M, V, C, n, a);
 }
 
 }  // namespace fx

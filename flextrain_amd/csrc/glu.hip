@@ -60,7 +60,7 @@ FX_DEV void glu_bwd_elem(float x1, float x3, float dout, float& dx1, float& dx3,
 constexpr int GLU_THREADS = 256;
 constexpr int GLU_UNROLL = 2;  // packs of 8 per lane
 
-template <typename T, typename TO, int ACT>
+template <typename T, typename TO, int ACT, bool NT>
 __global__ __launch_bounds__(GLU_THREADS) void glu_fwd_kernel(
     const T* __restrict__ X1, const T* __restrict__ X3, TO* __restrict__ OUT, int64_t n) {
     const int64_t base = ((int64_t)blockIdx.x * GLU_UNROLL) * GLU_THREADS * 8;
@@ -71,8 +71,8 @@ __global__ __launch_bounds__(GLU_THREADS) void glu_fwd_kernel(
         const int64_t off = base + ((int64_t)u * GLU_THREADS + threadIdx.x) * 8;
         full[u] = off + 8 <= n;
         if (full[u]) {
-            load_f32<T, 8>(X1 + off, a[u]);
-            load_f32<T, 8>(X3 + off, b[u]);
+            load_f32<T, 8, NT>(X1 + off, a[u]);
+            load_f32<T, 8, NT>(X3 + off, b[u]);
         }
     }
 #pragma unroll
@@ -82,7 +82,7 @@ __global__ __launch_bounds__(GLU_THREADS) void glu_fwd_kernel(
             float o[8];
 #pragma unroll
             for (int j = 0; j < 8; ++j) o[j] = glu_fwd_elem<T, ACT>(a[u][j], b[u][j]);
-            store_f32<TO, 8>(OUT + off, o);
+            store_f32<TO, 8, NT>(OUT + off, o);
         } else {
             for (int64_t i = off; i < n && i < off + 8; ++i)
                 OUT[i] = (TO)glu_fwd_elem<T, ACT>((float)X1[i], (float)X3[i]);
@@ -90,7 +90,7 @@ __global__ __launch_bounds__(GLU_THREADS) void glu_fwd_kernel(
     }
 }
 
-template <typename T, int ACT, bool STORE_ACT>
+template <typename T, int ACT, bool STORE_ACT, bool NT>
 __global__ __launch_bounds__(GLU_THREADS) void glu_bwd_kernel(
     const T* __restrict__ X1, const T* __restrict__ X3, const T* __restrict__ DOUT,
     T* __restrict__ DX1, T* __restrict__ DX3, T* __restrict__ ACTOUT, int64_t n) {
@@ -102,9 +102,9 @@ __global__ __launch_bounds__(GLU_THREADS) void glu_bwd_kernel(
         const int64_t off = base + ((int64_t)u * GLU_THREADS + threadIdx.x) * 8;
         full[u] = off + 8 <= n;
         if (full[u]) {
-            load_f32<T, 8>(X1 + off, a[u]);
-            load_f32<T, 8>(X3 + off, b[u]);
-            load_f32<T, 8>(DOUT + off, d[u]);
+            load_f32<T, 8, NT>(X1 + off, a[u]);
+            load_f32<T, 8, NT>(X3 + off, b[u]);
+            load_f32<T, 8, NT>(DOUT + off, d[u]);
         }
     }
 #pragma unroll
@@ -115,9 +115,9 @@ __global__ __launch_bounds__(GLU_THREADS) void glu_bwd_kernel(
 #pragma unroll
             for (int j = 0; j < 8; ++j)
                 glu_bwd_elem<T, ACT>(a[u][j], b[u][j], d[u][j], g1[j], g3[j], ac[j]);
-            store_f32<T, 8>(DX1 + off, g1);
-            store_f32<T, 8>(DX3 + off, g3);
-            if (STORE_ACT) store_f32<T, 8>(ACTOUT + off, ac);
+            store_f32<T, 8, NT>(DX1 + off, g1);
+            store_f32<T, 8, NT>(DX3 + off, g3);
+            if (STORE_ACT) store_f32<T, 8, NT>(ACTOUT + off, ac);
         } else {
             for (int64_t i = off; i < n && i < off + 8; ++i) {
                 float g1, g3, ac;
@@ -156,7 +156,11 @@ static void launch_glu_fwd(const void* x1, const void* x3, void* out, int64_t n,
     TO* o = reinterpret_cast<TO*>(out);
     if (aligned16(x1) && aligned16(x3) && aligned16(out)) {
         const int64_t per_block = (int64_t)GLU_UNROLL * GLU_THREADS * 8;
-        glu_fwd_kernel<T, TO, ACT><<<(unsigned)((n + per_block - 1) / per_block), GLU_THREADS, 0, s>>>(a, b, o, n);
+        const unsigned grid = (unsigned)((n + per_block - 1) / per_block);
+        if ((size_t)n * (2 * sizeof(T) + sizeof(TO)) >= kStreamingBytes)
+            glu_fwd_kernel<T, TO, ACT, true><<<grid, GLU_THREADS, 0, s>>>(a, b, o, n);
+        else
+            glu_fwd_kernel<T, TO, ACT, false><<<grid, GLU_THREADS, 0, s>>>(a, b, o, n);
     } else {
         glu_fwd_scalar_kernel<T, TO, ACT><<<(unsigned)((n + 255) / 256), 256, 0, s>>>(a, b, o, n);
     }
@@ -175,8 +179,11 @@ static void launch_glu_bwd(const void* x1, const void* x3, const void* dout, voi
         (act == nullptr || aligned16(act))) {
         const int64_t per_block = (int64_t)GLU_UNROLL * GLU_THREADS * 8;
         const unsigned grid = (unsigned)((n + per_block - 1) / per_block);
-        if (act) glu_bwd_kernel<T, ACT, true><<<grid, GLU_THREADS, 0, s>>>(a, b, d, g1, g3, ac, n);
-        else glu_bwd_kernel<T, ACT, false><<<grid, GLU_THREADS, 0, s>>>(a, b, d, g1, g3, ac, n);
+        const bool nt = (size_t)n * 5 * sizeof(T) >= kStreamingBytes;
+        if (act && nt) glu_bwd_kernel<T, ACT, true, true><<<grid, GLU_THREADS, 0, s>>>(a, b, d, g1, g3, ac, n);
+        else if (act) glu_bwd_kernel<T, ACT, true, false><<<grid, GLU_THREADS, 0, s>>>(a, b, d, g1, g3, ac, n);
+        else if (nt) glu_bwd_kernel<T, ACT, false, true><<<grid, GLU_THREADS, 0, s>>>(a, b, d, g1, g3, ac, n);
+        else glu_bwd_kernel<T, ACT, false, false><<<grid, GLU_THREADS, 0, s>>>(a, b, d, g1, g3, ac, n);
     } else {
         glu_bwd_scalar_kernel<T, ACT><<<(unsigned)((n + 255) / 256), 256, 0, s>>>(a, b, d, g1, g3, ac, n);
     }

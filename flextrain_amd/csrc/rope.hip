@@ -19,7 +19,7 @@ namespace fx {
 
 constexpr int ROPE_THREADS = 256;
 
-template <typename T, bool BWD>
+template <typename T, bool BWD, bool NT>
 __global__ __launch_bounds__(ROPE_THREADS) void rope_vec_kernel(
     T* __restrict__ Q, T* __restrict__ K, const int32_t* __restrict__ POS, int64_t stride_pos,
     const float* __restrict__ INV_FREQ, int64_t stride_if, int64_t T_tokens, int Hq, int Hk, int D,
@@ -52,14 +52,14 @@ __global__ __launch_bounds__(ROPE_THREADS) void rope_vec_kernel(
         T* p = (h < Hq) ? (Q + t * sq_t + (int64_t)h * sq_h) : (K + t * sk_t + (int64_t)(h - Hq) * sk_h);
         p += v * 8;
         float x[8], y[8];
-        load_f32<T, 8>(p, x);
+        load_f32<T, 8, NT>(p, x);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const float e = x[2 * j], o = x[2 * j + 1];
             y[2 * j] = e * c[j] - o * s[j];
             y[2 * j + 1] = e * s[j] + o * c[j];
         }
-        store_f32<T, 8>(p, y);
+        store_f32<T, 8, NT>(p, y);
     };
     if (tpt % vec_per_head == 0) {
         // Each lane keeps one pack position for every head: cos/sin stay in registers.
@@ -128,9 +128,15 @@ static int launch_rope(void* q, void* k, const int32_t* pos, int64_t stride_pos,
         while (tpb < 16 && items * tpb * 2 <= ROPE_THREADS) tpb *= 2;
         const size_t lds = (size_t)tpb * (rot_dim >> 1) * 2 * sizeof(float);
         const unsigned grid = (unsigned)((T_tokens + tpb - 1) / tpb);
-        rope_vec_kernel<T, BWD><<<grid, ROPE_THREADS, lds, s>>>(
-            Q, K, pos, stride_pos, inv_freq, stride_if, T_tokens, Hq, Hk, D, rot_dim, sq[0], sq[1],
-            Hk > 0 ? sk[0] : 0, Hk > 0 ? sk[1] : 0, tpb);
+        const bool nt = (size_t)T_tokens * (Hq + Hk) * rot_dim * sizeof(T) * 2 >= kStreamingBytes;
+        if (nt)
+            rope_vec_kernel<T, BWD, true><<<grid, ROPE_THREADS, lds, s>>>(
+                Q, K, pos, stride_pos, inv_freq, stride_if, T_tokens, Hq, Hk, D, rot_dim, sq[0], sq[1],
+                Hk > 0 ? sk[0] : 0, Hk > 0 ? sk[1] : 0, tpb);
+        else
+            rope_vec_kernel<T, BWD, false><<<grid, ROPE_THREADS, lds, s>>>(
+                Q, K, pos, stride_pos, inv_freq, stride_if, T_tokens, Hq, Hk, D, rot_dim, sq[0], sq[1],
+                Hk > 0 ? sk[0] : 0, Hk > 0 ? sk[1] : 0, tpb);
     } else {
         rope_generic_kernel<T, BWD><<<(unsigned)T_tokens, ROPE_THREADS, 0, s>>>(
             Q, K, pos, stride_pos, inv_freq, stride_if, Hq, Hk, rot_dim, sq[0], sq[1], sq[2],

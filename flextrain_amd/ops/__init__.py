@@ -9,6 +9,19 @@ from .glu import (
     flextrain_swiglu_bwd,
     flextrain_swiglu_fwd,
 )
+from .moe import (
+    flextrain_copy_expert_counts,
+    flextrain_fused_topk_softmax,
+    flextrain_load_balance_bwd,
+    flextrain_moe_gather,
+    flextrain_moe_router_gate_bwd,
+    flextrain_moe_scatter,
+    flextrain_moe_scatter_routing_weights,
+    flextrain_moe_sort,
+    flextrain_swiglu_moe_bwd,
+    flextrain_swiglu_moe_bwd_prescaled,
+    flextrain_swiglu_moe_fwd,
+)
 from .rmsnorm import (
     flextrain_rmsnorm_bwd,
     flextrain_rmsnorm_fwd,
@@ -25,6 +38,17 @@ from .rope import (
 __all__ = [
     "build_rope_inv_freq",
     "flextrain_adamw_step",
+    "flextrain_copy_expert_counts",
+    "flextrain_fused_topk_softmax",
+    "flextrain_load_balance_bwd",
+    "flextrain_moe_gather",
+    "flextrain_moe_router_gate_bwd",
+    "flextrain_moe_scatter",
+    "flextrain_moe_scatter_routing_weights",
+    "flextrain_moe_sort",
+    "flextrain_swiglu_moe_bwd",
+    "flextrain_swiglu_moe_bwd_prescaled",
+    "flextrain_swiglu_moe_fwd",
     "flextrain_gelu_tanh_gated_bwd",
     "flextrain_gelu_tanh_gated_fwd",
     "flextrain_rmsnorm_bwd",

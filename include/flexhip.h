@@ -112,6 +112,78 @@ int fx_adamw_step(void* p, const void* g, void* m, void* v, void* p_bf16_out, in
  * caller-zeroed) if any element of x is NaN or infinite. */
 int fx_nonfinite_flag(const void* x, int64_t n, int dt, int* flag, hipStream_t stream);
 
+/* ---- MoE routing --------------------------------------------------------- */
+
+/* flextrain_fused_topk_softmax (flextrain/ops/_kernels/moe.py:848-943; kernel
+ * :218-314).  logits (T,E) contiguous; ids_out int32 (T,K); weights_out (T,K)
+ * of dtype weights_dt.  mode 0 = topk_then_softmax, 1 = softmax_then_topk.
+ * Ties go to the smallest expert index; slots are in descending value order. */
+int fx_topk_softmax(const void* logits, int32_t* ids_out, void* weights_out, int64_t T, int E, int K,
+                    int logits_dt, int weights_dt, int mode, hipStream_t stream);
+
+/* Scratch bytes for fx_moe_sort (replaces block_counts / block_accum /
+ * total_counts / expert_starts / offsets, flextrain/ops/_kernels/moe.py:679-758). */
+size_t fx_moe_sort_ws_bytes(int64_t n_pairs, int E);
+
+/* flextrain_moe_sort (flextrain/ops/_kernels/moe.py:649-783) fused with
+ * flextrain_copy_expert_counts (:787-834).  ids: n_pairs = T*K flat expert ids
+ * (int32, or int64 when ids_are_int64).  index_out[i] = row of pair i in the
+ * expert-grouped order (stable).  counts_out (device, E int32) and counts_host
+ * (pinned host memory mapped into the device, E int32) are optional. */
+int fx_moe_sort(const void* ids, int ids_are_int64, int64_t n_pairs, int E, void* index_out,
+                int index_is_int64, int32_t* counts_out, int32_t* counts_host, void* ws, size_t ws_bytes,
+                hipStream_t stream);
+
+/* flextrain_copy_expert_counts (flextrain/ops/_kernels/moe.py:787-834; kernel
+ * :498-505): a kernel copies n int32 from device memory to dst, which may be
+ * pinned host memory (zero-copy store). */
+int fx_copy_i32(const int32_t* src_dev, int32_t* dst, int n, hipStream_t stream);
+
+/* flextrain_moe_router_gate_bwd (flextrain/ops/_kernels/moe.py:1527-1655;
+ * kernel :360-458).  dlogits (T,E) is accumulated into.  dprobs is indexed
+ * through indices (T,K); probs (T,K); logits (T,E) only for mode 1. */
+int fx_router_gate_bwd(void* dlogits, const void* dprobs, const void* probs, const void* indices,
+                       int indices_are_int64, const int32_t* chosen_experts, const void* logits, int64_t T,
+                       int K, int E, int dt, int dprobs_dt, int mode, hipStream_t stream);
+
+/* flextrain_load_balance_bwd (flextrain/ops/_kernels/moe.py:1658-1745; kernel
+ * :601-642).  dlogits += scale * p * (f - <f,p>), f = counts / (T*top_k);
+ * scale = alpha*E/tokens_per_step is computed by the caller. */
+int fx_load_balance_bwd(const void* logits, const int32_t* expert_counts, void* dlogits, int64_t T, int E,
+                        int top_k, float scale, int logits_dt, int dlogits_dt, hipStream_t stream);
+
+/* ---- MoE data movement and expert activation ----------------------------- */
+
+/* flextrain_moe_scatter (flextrain/ops/_kernels/moe.py:946-1050; kernel :508-543).
+ * x (T,D) contiguous; out row r starts at out + r*out_row_stride; scales (T,K)
+ * optional, in original (token, slot) order. */
+int fx_moe_scatter(const void* x, const void* indices, int indices_are_int64, const void* scales,
+                   int scales_dt, void* out, int64_t T, int D, int K, int64_t out_row_stride, int dt,
+                   hipStream_t stream);
+
+/* flextrain_moe_scatter_routing_weights (flextrain/ops/_kernels/moe.py:1053-1127). */
+int fx_moe_scatter_weights(const void* weights, const void* indices, int indices_are_int64, void* out,
+                           int64_t n, int dt, hipStream_t stream);
+
+/* flextrain_moe_gather (flextrain/ops/_kernels/moe.py:1130-1271; kernel :560-598).
+ * expert_out (T*K,D) contiguous; weights (T,K) and residual (T,D) optional;
+ * fp32 accumulation, residual first, k ascending. */
+int fx_moe_gather(const void* expert_out, const void* indices, int indices_are_int64, const void* weights,
+                  int weights_dt, const void* residual, int residual_dt, void* out, int out_dt, int64_t T,
+                  int D, int K, int dt, hipStream_t stream);
+
+/* flextrain_swiglu_moe_fwd (flextrain/ops/_kernels/moe.py:1274-1320; kernel :29-74).
+ * x rows are packed [value (F) | gate (F)]; w (rows,) optional. */
+int fx_swiglu_moe_fwd(const void* x, const void* w, int w_dt, void* out, int out_dt, int64_t rows, int F,
+                      int64_t x_row_stride, int64_t out_row_stride, int dt, hipStream_t stream);
+
+/* flextrain_swiglu_moe_bwd and flextrain_swiglu_moe_bwd_prescaled
+ * (flextrain/ops/_kernels/moe.py:1323-1524; kernels :77-215).  dx rows are
+ * packed [d value | d gate]; dw (rows,) receives sum_F dout*act; fwd_act optional. */
+int fx_swiglu_moe_bwd(void* dx, void* dw, int dw_dt, const void* dout, const void* x, const void* w, int w_dt,
+                      void* fwd_act, int64_t rows, int F, int64_t dx_row_stride, int64_t dout_row_stride,
+                      int64_t x_row_stride, int64_t act_row_stride, int dt, int prescaled, hipStream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,5 +1,7 @@
 """HIP AdamW against the CPU oracle: fp32 parameters and optimizer state at
-rtol 1e-4 (atol 1e-9 for p, 1e-12 / 1e-15 for m / v, far below their scale);
+rtol 1e-4; the absolute floors (p 1e-9, m 1e-8, v 1e-12) are 1e-4 of each
+quantity's typical magnitude here (p ~2e-2, m ~1e-4, v ~5e-8) and only matter
+where beta*m and (1-beta)*g cancel;
 bf16 state at rtol = atol = 1e-2."""
 import pytest
 import torch
@@ -26,8 +28,8 @@ def test_fp32_master_four_steps(dev, n):
         rc = ops.flextrain_adamw_step(pd, grad.to(dev), md, vd, step=step, params_bf16_out=pb, **HP)
         assert rc == 0
         close(pd, p, rtol=1e-4, atol=1e-9, what=f"p step {step}")
-        close(md, m, rtol=1e-4, atol=1e-12, what=f"m step {step}")
-        close(vd, v, rtol=1e-4, atol=1e-15, what=f"v step {step}")
+        close(md, m, rtol=1e-4, atol=1e-8, what=f"m step {step}")
+        close(vd, v, rtol=1e-4, atol=1e-12, what=f"v step {step}")
         close(pb, pbf, rtol=1e-2, atol=1e-2, what="bf16 copy")
         assert torch.equal(pb, pd.to(torch.bfloat16))
 
