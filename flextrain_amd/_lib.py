@@ -7,7 +7,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import c_char_p, c_float, c_int, c_int32, c_int64, c_size_t, c_void_p, POINTER
+from ctypes import c_char_p, c_float, c_int, c_int32, c_int64, c_size_t, c_uint64, c_void_p, POINTER
 
 import torch
 
@@ -64,6 +64,19 @@ _SIGNATURES = {
                               c_int64, c_int, c_int, c_int, c_void_p]),
     "fx_swiglu_moe_fwd": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int64, c_int, c_int64,
                                   c_int64, c_int, c_void_p]),
+    "fx_grouped_ws_bytes": (c_size_t, [c_int, c_int64]),
+    "fx_grouped_gemm_rows": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int, c_void_p, c_int64,
+                                     c_void_p, c_int64, c_void_p, c_int, c_int64, c_int, c_int, c_float, c_float,
+                                     c_int, c_void_p, c_size_t, c_void_p]),
+    "fx_grouped_gemm_wgrad": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int,
+                                      c_void_p, c_int, c_int64, c_int, c_int, c_float, c_float, c_int, c_void_p,
+                                      c_size_t, c_void_p]),
+    "create_dispatcher": (c_void_p, [c_int, c_int]),
+    "destroy_dispatcher": (None, [c_void_p]),
+    "get_stats": (None, [c_void_p, POINTER(c_uint64)]),
+    "dispatch_matmul": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int,
+                                c_void_p, c_int, c_void_p, c_int, c_void_p, c_size_t, c_int, c_int, c_int,
+                                c_int, c_int, c_float, c_float, c_int, c_int]),
     "fx_swiglu_moe_bwd": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                   c_int64, c_int, c_int64, c_int64, c_int64, c_int64, c_int, c_int,
                                   c_void_p]),

@@ -1,0 +1,261 @@
+// Strided row-major GEMM with the reference dispatcher's C ABI, gfx950.
+//
+//   D = alpha * op(A) * op(B) + beta * C,  fp32 accumulation, row-major storage.
+//
+// Stands in for helpers/matmul_dispatcher/src/dispatch.cpp:113-323
+// (create_dispatcher / destroy_dispatcher / get_stats / dispatch_matmul).  The
+// reference asks cuBLASLt for an algorithm and caches it per exact shape and per
+// rounded ("fuzzy") shape; here the cached "algorithm" is the tile shape of the
+// hand-written MFMA kernel in gemm_core.h, chosen by a fill heuristic, and the
+// cache/statistics bookkeeping keeps the same meaning (exact hit, fuzzy hit,
+// new algorithm saved).
+#include <chrono>
+#include <unordered_map>
+
+#include "gemm_core.h"
+#include "flexhip.h"
+
+namespace fx {
+
+// blockIdx.x -> (tile_m, tile_n).  Workgroups are dealt round-robin to the 8 XCDs,
+// each with its own L2: give every XCD a contiguous band of tile indices and walk
+// the band in groups of GROUP_M tile-rows so concurrently resident workgroups
+// share A rows and B columns in L2.
+FX_DEV void tile_coords(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
+    const int total = tiles_m * tiles_n;
+    constexpr int XCDS = 8;
+    int p = pid;
+    if (total >= XCDS * 4) {
+        const int per = total / XCDS;          // band length; the remainder keeps its order
+        const int body = per * XCDS;
+        if (pid < body) p = (pid % XCDS) * per + pid / XCDS;
+    }
+    constexpr int GROUP_M = 8;
+    const int width = GROUP_M * tiles_n;
+    const int group = p / width;
+    const int first_m = group * GROUP_M;
+    const int gsz = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
+    tm = first_m + (p % width) % gsz;
+    tn = (p % width) / gsz;
+}
+
+template <typename T, typename TD, int BM, int BN, bool A_MN, bool B_MN>
+__global__ __launch_bounds__(GEMM_THREADS) void gemm_kernel(
+    const T* __restrict__ A, const T* __restrict__ B, const TD* C, TD* D, int M, int N, int K, int64_t lda,
+    int64_t ldb, int64_t ldc, int64_t ldd, float alpha, float beta, int tiles_m, int tiles_n) {
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T* smem = reinterpret_cast<T*>(smem_raw);
+    int tm, tn;
+    tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
+    OperandView<T> a{A, lda, M, tm * BM};
+    OperandView<T> b{B, ldb, N, tn * BN};
+    gemm_tile<T, TD, BM, BN, A_MN, B_MN>(a, b, C, D, ldc, ldd, M, N, K, 0, alpha, beta, smem);
+}
+
+// Any dtype / alignment: one output element per lane.  Correct, not fast.
+template <typename TA, typename TB, typename TC, typename TD>
+__global__ __launch_bounds__(256) void gemm_generic_kernel(
+    const TA* __restrict__ A, const TB* __restrict__ B, const TC* C, TD* D, int M, int N, int K, int64_t lda,
+    int64_t ldb, int64_t ldc, int64_t ldd, float alpha, float beta, int ta, int tb) {
+    const int n = blockIdx.x * 16 + (threadIdx.x & 15);
+    const int m = blockIdx.y * 16 + (threadIdx.x >> 4);
+    if (m >= M || n >= N) return;
+    float acc = 0.f;
+    for (int k = 0; k < K; ++k) {
+        const float a = (float)(ta ? A[(int64_t)k * lda + m] : A[(int64_t)m * lda + k]);
+        const float b = (float)(tb ? B[(int64_t)n * ldb + k] : B[(int64_t)k * ldb + n]);
+        acc += a * b;
+    }
+    float r = alpha * acc;
+    if (beta != 0.f) r += beta * (float)C[(int64_t)m * ldc + n];
+    D[(int64_t)m * ldd + n] = (TD)r;
+}
+
+enum TileCfg : int { TILE_256x256 = 0, TILE_256x128 = 1, TILE_128x128 = 2, TILE_GENERIC = 3 };
+
+static inline int cdiv(int a, int b) { return (a + b - 1) / b; }
+
+// Largest tile that still gives every CU at least one workgroup.
+static TileCfg choose_tile(int M, int N) {
+    const long cus = 256;
+    if ((long)cdiv(M, 256) * cdiv(N, 256) >= cus) return TILE_256x256;
+    if ((long)cdiv(M, 256) * cdiv(N, 128) >= cus) return TILE_256x128;
+    return TILE_128x128;
+}
+
+template <typename T, typename TD, int BM, int BN>
+static void launch_tile(const void* A, const void* B, const void* C, void* D, int M, int N, int K, int64_t lda,
+                        int64_t ldb, int64_t ldc, int64_t ldd, float alpha, float beta, int ta, int tb,
+                        hipStream_t s) {
+    const int tiles_m = cdiv(M, BM), tiles_n = cdiv(N, BN);
+    const unsigned grid = (unsigned)(tiles_m * tiles_n);
+    const size_t lds = (size_t)(BM + BN) * GEMM_BK * sizeof(T);
+    const T* a = reinterpret_cast<const T*>(A);
+    const T* b = reinterpret_cast<const T*>(B);
+    const TD* c = reinterpret_cast<const TD*>(C);
+    TD* d = reinterpret_cast<TD*>(D);
+    // operand form: A is MN-contiguous when transposed, B when NOT transposed
+#define FX_GEMM_GO(AM, BMN) gemm_kernel<T, TD, BM, BN, AM, BMN><<<grid, GEMM_THREADS, lds, s>>>(a, b, c, d, M, N, K, lda, ldb, ldc, ldd, alpha, beta, tiles_m, tiles_n)
+    if (!ta && tb) FX_GEMM_GO(false, false);
+    else if (!ta && !tb) FX_GEMM_GO(false, true);
+    else if (ta && tb) FX_GEMM_GO(true, false);
+    else FX_GEMM_GO(true, true);
+#undef FX_GEMM_GO
+}
+
+template <typename T, typename TD>
+static void launch_cfg(TileCfg cfg, const void* A, const void* B, const void* C, void* D, int M, int N, int K,
+                       int64_t lda, int64_t ldb, int64_t ldc, int64_t ldd, float alpha, float beta, int ta,
+                       int tb, hipStream_t s) {
+    if (cfg == TILE_256x256) launch_tile<T, TD, 256, 256>(A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, ta, tb, s);
+    else if (cfg == TILE_256x128) launch_tile<T, TD, 256, 128>(A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, ta, tb, s);
+    else launch_tile<T, TD, 128, 128>(A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, ta, tb, s);
+}
+
+// Can the MFMA path take this problem?  16-byte aligned operands whose
+// contiguous axis is a multiple of 8 elements.
+static bool mfma_ok(const void* A, const void* B, int M, int N, int K, int64_t lda, int64_t ldb, int a_dt,
+                    int b_dt, int c_dt, int d_dt, int ta, int tb, bool has_c) {
+    if (a_dt != b_dt || (a_dt != DT_BF16 && a_dt != DT_F16)) return false;
+    if (d_dt != a_dt && !(a_dt == DT_BF16 && d_dt == DT_F32)) return false;
+    if (has_c && c_dt != d_dt) return false;
+    if (!aligned16(A) || !aligned16(B) || (lda & 7) || (ldb & 7)) return false;
+    if (ta ? (M & 7) : (K & 7)) return false;
+    if (tb ? (K & 7) : (N & 7)) return false;
+    return true;
+}
+
+struct ShapeKey {
+    int M, N, K, lda, ldb, ldc, ldd, a_dt, b_dt, c_dt, d_dt, ta, tb;
+    bool operator==(const ShapeKey& o) const {
+        return M == o.M && N == o.N && K == o.K && lda == o.lda && ldb == o.ldb && ldc == o.ldc && ldd == o.ldd &&
+               a_dt == o.a_dt && b_dt == o.b_dt && c_dt == o.c_dt && d_dt == o.d_dt && ta == o.ta && tb == o.tb;
+    }
+};
+struct ShapeHash {
+    size_t operator()(const ShapeKey& k) const {
+        size_t h = 1469598103934665603ull;
+        const int* p = reinterpret_cast<const int*>(&k);
+        for (size_t i = 0; i < sizeof(ShapeKey) / sizeof(int); ++i) h = (h ^ (size_t)(unsigned)p[i]) * 1099511628211ull;
+        return h;
+    }
+};
+
+}  // namespace fx
+
+using namespace fx;
+
+// Opaque to callers (helpers/matmul_dispatcher/src/dispatch.h:12).
+struct DispatchContext {
+    int round_multiple;
+    int max_algos;
+    std::unordered_map<ShapeKey, int, ShapeHash> exact;   // full problem -> tile config
+    std::unordered_map<ShapeKey, int, ShapeHash> fuzzy;   // dims rounded up to round_multiple
+    uint64_t algos_saved = 0, calls = 0, hits = 0, total_ns = 0, hash_ns = 0, lookup_ns = 0, driver_ns = 0;
+};
+
+static inline uint64_t now_ns() {
+    return (uint64_t)std::chrono::duration_cast<std::chrono::nanoseconds>(
+               std::chrono::steady_clock::now().time_since_epoch()).count();
+}
+
+extern "C" DispatchContext* create_dispatcher(int round_multiple, int max_algos) {
+    DispatchContext* ctx = new DispatchContext();
+    ctx->round_multiple = round_multiple > 0 ? round_multiple : 1;
+    ctx->max_algos = max_algos;
+    return ctx;
+}
+
+extern "C" void destroy_dispatcher(DispatchContext* ctx) { delete ctx; }
+
+// out_stats[7] = {algos_saved, calls, hits, total_ns, hash_ns, lookup_ns, driver_ns}
+// (helpers/matmul_dispatcher/src/dispatch.cpp:138-147).
+extern "C" void get_stats(DispatchContext* ctx, uint64_t* out_stats) {
+    if (!ctx || !out_stats) return;
+    out_stats[0] = ctx->algos_saved;
+    out_stats[1] = ctx->calls;
+    out_stats[2] = ctx->hits;
+    out_stats[3] = ctx->total_ns;
+    out_stats[4] = ctx->hash_ns;
+    out_stats[5] = ctx->lookup_ns;
+    out_stats[6] = ctx->driver_ns;
+}
+
+static int round_up(int v, int m) { return (v + m - 1) / m * m; }
+
+extern "C" int dispatch_matmul(DispatchContext* ctx, intptr_t stream_ptr, int M, int N, int K, intptr_t ptr_A,
+                               int lda, intptr_t ptr_B, int ldb, intptr_t ptr_C, int ldc, intptr_t ptr_D,
+                               int ldd, intptr_t ptr_workspace, size_t workspace_bytes, int a_dt, int b_dt,
+                               int c_dt, int d_dt, int compute_dt, float alpha, float beta, int trans_a,
+                               int trans_b) {
+    (void)ptr_workspace; (void)workspace_bytes; (void)compute_dt;  // fp32 compute always; no workspace needed
+    const uint64_t t0 = now_ns();
+    if (M == 0 || N == 0 || K == 0) return 0;  // no-op, as the reference (dispatch.cpp:161)
+    if (!ctx) FX_FAIL("dispatch_matmul: null dispatcher");
+    if (M < 0 || N < 0 || K < 0) FX_FAIL("dispatch_matmul: negative dimension");
+    if (!ptr_A || !ptr_B || !ptr_D) FX_FAIL("dispatch_matmul: null operand");
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_ptr);
+    const void* A = reinterpret_cast<const void*>(ptr_A);
+    const void* B = reinterpret_cast<const void*>(ptr_B);
+    const void* C = reinterpret_cast<const void*>(ptr_C);
+    void* D = reinterpret_cast<void*>(ptr_D);
+    const bool has_c = (C != nullptr) && beta != 0.f;
+    if (!has_c) beta = 0.f;
+
+    ctx->calls++;
+    const uint64_t h0 = now_ns();
+    ShapeKey key{M, N, K, lda, ldb, ldc, ldd, a_dt, b_dt, c_dt, d_dt, trans_a, trans_b};
+    const uint64_t h1 = now_ns();
+    int cfg;
+    auto it = ctx->exact.find(key);
+    if (it != ctx->exact.end()) {
+        cfg = it->second;
+        ctx->hits++;
+    } else {
+        const int r = ctx->round_multiple;
+        ShapeKey fk{round_up(M, r), round_up(N, r), round_up(K, r), 0, 0, 0, 0, a_dt, b_dt, c_dt, d_dt, trans_a, trans_b};
+        const bool fast = mfma_ok(A, B, M, N, K, lda, ldb, a_dt, b_dt, c_dt, d_dt, trans_a, trans_b, has_c);
+        auto fit = ctx->fuzzy.find(fk);
+        if (!fast) {
+            cfg = TILE_GENERIC;
+        } else if (fit != ctx->fuzzy.end() && fit->second != TILE_GENERIC) {
+            cfg = fit->second;
+            ctx->hits++;
+        } else {
+            cfg = choose_tile(M, N);
+            ctx->fuzzy[fk] = cfg;
+            ctx->algos_saved++;
+        }
+        ctx->exact[key] = cfg;
+    }
+    const uint64_t h2 = now_ns();
+
+    if (cfg == TILE_GENERIC) {
+        dim3 grid((unsigned)cdiv(N, 16), (unsigned)cdiv(M, 16));
+        const int cdt = has_c ? c_dt : d_dt;
+        if (cdt != d_dt) FX_FAIL("dispatch_matmul: C and D must share a dtype");
+        if (a_dt != b_dt) FX_FAIL("dispatch_matmul: A and B must share a dtype");
+        FX_DISPATCH_DTYPE(a_dt, TA,
+            FX_DISPATCH_DTYPE(d_dt, TD,
+                gemm_generic_kernel<TA, TA, TD, TD><<<grid, 256, 0, stream>>>(
+                    reinterpret_cast<const TA*>(A), reinterpret_cast<const TA*>(B), reinterpret_cast<const TD*>(C),
+                    reinterpret_cast<TD*>(D), M, N, K, lda, ldb, ldc, ldd, alpha, beta, trans_a, trans_b)));
+    } else if (a_dt == DT_BF16 && d_dt == DT_BF16) {
+        launch_cfg<bf16, bf16>((TileCfg)cfg, A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, trans_a, trans_b, stream);
+    } else if (a_dt == DT_BF16) {
+        launch_cfg<bf16, float>((TileCfg)cfg, A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, trans_a, trans_b, stream);
+    } else {
+        launch_cfg<f16, f16>((TileCfg)cfg, A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, trans_a, trans_b, stream);
+    }
+    const uint64_t h3 = now_ns();
+    ctx->hash_ns += h1 - h0;
+    ctx->lookup_ns += h2 - h1;
+    ctx->driver_ns += h3 - h2;
+    ctx->total_ns += h3 - t0;
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        fprintf(stderr, "flexhip: dispatch_matmul launch failed: %s\n", hipGetErrorString(e));
+        return -1;
+    }
+    return 0;
+}

@@ -1,0 +1,186 @@
+// Expert-grouped GEMMs for the MoE block, gfx950.
+//
+// The reference runs a Python loop over experts, one cuBLASLt call per GEMM, after
+// copying the per-expert row counts to the host and synchronising
+// (flextrain/ops/full_moe.py:144-148, :428-466, :545-626).  Here each GEMM family
+// is ONE launch whose workgroups find their expert from the counts that are still
+// on the device, so no host round trip is needed:
+//
+//   rows form   D_e[c_e, N]  = alpha * A_e[c_e, K] * op(B[e]) + beta * C_e      (up / down / dgrad)
+//   wgrad form  G[e][M, N]   = alpha * A_e[c_e, M]^T * B_e[c_e, N] + beta * G[e]
+//
+// where rows of expert e are the contiguous range [off_e, off_e + c_e) of the
+// expert-sorted buffers and off = exclusive prefix sum of the counts.
+#include "gemm_core.h"
+#include "flexhip.h"
+
+namespace fx {
+
+// Workspace layout (int32): [0] number of tiles, [1 .. E+1] row offsets (E+1 entries),
+// then (expert, first_row_in_expert) pairs, one per BM-row tile.
+struct GroupedWs {
+    int32_t* ntiles;
+    int32_t* offsets;
+    int32_t* tiles;
+};
+
+static inline GroupedWs split_ws(void* ws, int E) {
+    int32_t* p = reinterpret_cast<int32_t*>(ws);
+    return GroupedWs{p, p + 1, p + 2 + E};
+}
+
+__global__ __launch_bounds__(256) void grouped_plan_kernel(const int32_t* __restrict__ COUNTS, int E, int BM,
+                                                           int32_t* __restrict__ NTILES,
+                                                           int32_t* __restrict__ OFFSETS,
+                                                           int32_t* __restrict__ TILES) {
+    __shared__ int32_t wsum_r[4], wsum_t[4];
+    __shared__ int32_t carry_r, carry_t;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (threadIdx.x == 0) { carry_r = 0; carry_t = 0; }
+    __syncthreads();
+    for (int base = 0; base < E; base += 256) {
+        const int e = base + threadIdx.x;
+        const int32_t c = e < E ? COUNTS[e] : 0;
+        const int32_t nt = (c + BM - 1) / BM;
+        int32_t ir = c, it = nt;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int32_t orr = __shfl_up(ir, off, 64);
+            const int32_t ot = __shfl_up(it, off, 64);
+            if (lane >= off) { ir += orr; it += ot; }
+        }
+        if (lane == 63) { wsum_r[wave] = ir; wsum_t[wave] = it; }
+        __syncthreads();
+        int32_t br = carry_r, bt = carry_t;
+        for (int w = 0; w < wave; ++w) { br += wsum_r[w]; bt += wsum_t[w]; }
+        if (e < E) {
+            OFFSETS[e] = br + ir - c;
+            const int32_t first = bt + it - nt;
+            for (int32_t t = 0; t < nt; ++t) {
+                TILES[2 * (first + t)] = e;
+                TILES[2 * (first + t) + 1] = t * BM;
+            }
+        }
+        __syncthreads();
+        if (threadIdx.x == 255) { carry_r = br + ir; carry_t = bt + it; }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) { OFFSETS[E] = carry_r; NTILES[0] = carry_t; }
+}
+
+template <typename T, int BM, int BN, bool B_MN>
+__global__ __launch_bounds__(GEMM_THREADS) void grouped_rows_kernel(
+    const T* __restrict__ A, int64_t lda, const T* __restrict__ B, int64_t ldb, int64_t b_expert_stride,
+    const T* C, int64_t ldc, T* D, int64_t ldd, const int32_t* __restrict__ NTILES,
+    const int32_t* __restrict__ OFFSETS, const int32_t* __restrict__ TILES, int N, int K, float alpha,
+    float beta) {
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T* smem = reinterpret_cast<T*>(smem_raw);
+    const int tile = blockIdx.x;
+    if (tile >= NTILES[0]) return;  // the grid is sized for the worst case
+    const int e = TILES[2 * tile];
+    const int m0 = TILES[2 * tile + 1];
+    const int64_t row0 = OFFSETS[e];
+    const int rows = OFFSETS[e + 1] - OFFSETS[e];
+    OperandView<T> a{A + row0 * lda, lda, rows, m0};
+    OperandView<T> b{B + (int64_t)e * b_expert_stride, ldb, N, (int)blockIdx.y * BN};
+    const T* c = C ? C + row0 * ldc : nullptr;
+    gemm_tile<T, T, BM, BN, false, B_MN>(a, b, c, D + row0 * ldd, ldc, ldd, rows, N, K, 0, alpha, beta, smem);
+}
+
+template <typename T, typename TG, int BM, int BN>
+__global__ __launch_bounds__(GEMM_THREADS) void grouped_wgrad_kernel(
+    const T* __restrict__ A, int64_t lda, const T* __restrict__ B, int64_t ldb, TG* G, int64_t ldg,
+    int64_t g_expert_stride, const int32_t* __restrict__ OFFSETS, int M, int N, float alpha, float beta,
+    int tiles_n) {
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T* smem = reinterpret_cast<T*>(smem_raw);
+    const int e = blockIdx.y;
+    const int64_t row0 = OFFSETS[e];
+    const int rows = OFFSETS[e + 1] - OFFSETS[e];
+    if (rows == 0 && beta == 1.f) return;  // nothing to add
+    const int tm = blockIdx.x / tiles_n, tn = blockIdx.x % tiles_n;
+    OperandView<T> a{A + row0 * lda, lda, M, tm * BM};
+    OperandView<T> b{B + row0 * ldb, ldb, N, tn * BN};
+    TG* g = G + (int64_t)e * g_expert_stride;
+    gemm_tile<T, TG, BM, BN, true, true>(a, b, g, g, ldg, ldg, M, N, rows, 0, alpha, beta, smem);
+}
+
+static inline int cdiv_i(int64_t a, int b) { return (int)((a + b - 1) / b); }
+
+}  // namespace fx
+
+using namespace fx;
+
+extern "C" size_t fx_grouped_ws_bytes(int E, int64_t total_rows) {
+    if (E <= 0 || total_rows < 0) return 0;
+    // smallest row tile is 128: at most total_rows/128 + E tiles
+    return sizeof(int32_t) * (size_t)(2 + E + 2 * (total_rows / 128 + E + 1));
+}
+
+static int rows_bm(int64_t total_rows, int E) { return (total_rows / (E > 0 ? E : 1)) >= 1024 ? 256 : 128; }
+
+extern "C" int fx_grouped_gemm_rows(const void* A, int64_t lda, const void* B, int64_t ldb,
+                                    int64_t b_expert_stride, int trans_b, const void* C, int64_t ldc, void* D,
+                                    int64_t ldd, const int32_t* counts, int E, int64_t total_rows, int N, int K,
+                                    float alpha, float beta, int dt, void* ws, size_t ws_bytes,
+                                    hipStream_t stream) {
+    if (E <= 0 || total_rows < 0 || N <= 0 || K <= 0) FX_FAIL("fx_grouped_gemm_rows: bad shape");
+    if (total_rows == 0) return 0;
+    if (!A || !B || !D || !counts) FX_FAIL("fx_grouped_gemm_rows: null pointer");
+    if (!ws || ws_bytes < fx_grouped_ws_bytes(E, total_rows)) FX_FAIL("fx_grouped_gemm_rows: workspace too small");
+    if (dt != DT_BF16 && dt != DT_F16) FX_FAIL("fx_grouped_gemm_rows: bf16 or fp16 only");
+    if (!aligned16(A) || !aligned16(B) || !aligned16(D) || (lda & 7) || (ldb & 7) || (K & 7) || (b_expert_stride & 7) ||
+        (!trans_b && (N & 7)))
+        FX_FAIL("fx_grouped_gemm_rows: operands must be 16-byte aligned with K (and N when B is (K,N)) a multiple of 8");
+    if (!C || beta == 0.f) { C = nullptr; beta = 0.f; }
+    GroupedWs w = split_ws(ws, E);
+    const int BM = rows_bm(total_rows, E);
+    grouped_plan_kernel<<<1, 256, 0, stream>>>(counts, E, BM, w.ntiles, w.offsets, w.tiles);
+    FX_CHECK_LAUNCH("fx_grouped_gemm_rows(plan)");
+    const unsigned max_tiles = (unsigned)(total_rows / BM + E);
+#define FX_ROWS(TT, BM_, BN_, BMN)                                                                        \
+    grouped_rows_kernel<TT, BM_, BN_, BMN><<<dim3(max_tiles, (unsigned)cdiv_i(N, BN_)), GEMM_THREADS,     \
+                                            (size_t)(BM_ + BN_) * GEMM_BK * sizeof(TT), stream>>>(         \
+        reinterpret_cast<const TT*>(A), lda, reinterpret_cast<const TT*>(B), ldb, b_expert_stride,        \
+        reinterpret_cast<const TT*>(C), ldc, reinterpret_cast<TT*>(D), ldd, w.ntiles, w.offsets, w.tiles, N, K, \
+        alpha, beta)
+#define FX_ROWS_T(TT)                                                                                     \
+    if (BM == 256) { if (trans_b) FX_ROWS(TT, 256, 256, false); else FX_ROWS(TT, 256, 256, true); }      \
+    else { if (trans_b) FX_ROWS(TT, 128, 256, false); else FX_ROWS(TT, 128, 256, true); }
+    if (dt == DT_BF16) { FX_ROWS_T(bf16) } else { FX_ROWS_T(f16) }
+#undef FX_ROWS_T
+#undef FX_ROWS
+    FX_CHECK_LAUNCH("fx_grouped_gemm_rows");
+    return 0;
+}
+
+extern "C" int fx_grouped_gemm_wgrad(const void* A, int64_t lda, const void* B, int64_t ldb, void* G, int64_t ldg,
+                                     int64_t g_expert_stride, int g_dt, const int32_t* counts, int E,
+                                     int64_t total_rows, int M, int N, float alpha, float beta, int dt, void* ws,
+                                     size_t ws_bytes, hipStream_t stream) {
+    if (E <= 0 || total_rows < 0 || M <= 0 || N <= 0) FX_FAIL("fx_grouped_gemm_wgrad: bad shape");
+    if (!A || !B || !G || !counts) FX_FAIL("fx_grouped_gemm_wgrad: null pointer");
+    if (!ws || ws_bytes < fx_grouped_ws_bytes(E, total_rows)) FX_FAIL("fx_grouped_gemm_wgrad: workspace too small");
+    if (dt != DT_BF16 && dt != DT_F16) FX_FAIL("fx_grouped_gemm_wgrad: bf16 or fp16 only");
+    if (g_dt != dt && !(dt == DT_BF16 && g_dt == DT_F32)) FX_FAIL("fx_grouped_gemm_wgrad: G must match the inputs or be fp32 (bf16 inputs)");
+    if (!aligned16(A) || !aligned16(B) || (lda & 7) || (ldb & 7) || (M & 7) || (N & 7))
+        FX_FAIL("fx_grouped_gemm_wgrad: operands must be 16-byte aligned with M and N multiples of 8");
+    GroupedWs w = split_ws(ws, E);
+    grouped_plan_kernel<<<1, 256, 0, stream>>>(counts, E, 128, w.ntiles, w.offsets, w.tiles);
+    FX_CHECK_LAUNCH("fx_grouped_gemm_wgrad(plan)");
+    constexpr int BM = 256, BN = 256;
+    const int tiles_m = cdiv_i(M, BM), tiles_n = cdiv_i(N, BN);
+    const dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)E);
+    const size_t lds = (size_t)(BM + BN) * GEMM_BK * 2;
+#define FX_WG(TT, TG)                                                                                     \
+    grouped_wgrad_kernel<TT, TG, BM, BN><<<grid, GEMM_THREADS, lds, stream>>>(                            \
+        reinterpret_cast<const TT*>(A), lda, reinterpret_cast<const TT*>(B), ldb, reinterpret_cast<TG*>(G), ldg, \
+        g_expert_stride, w.offsets, M, N, alpha, beta, tiles_n)
+    if (dt == DT_BF16 && g_dt == DT_BF16) FX_WG(bf16, bf16);
+    else if (dt == DT_BF16) FX_WG(bf16, float);
+    else FX_WG(f16, f16);
+#undef FX_WG
+    FX_CHECK_LAUNCH("fx_grouped_gemm_wgrad");
+    return 0;
+}

@@ -1,0 +1,212 @@
+"""Routed-SwiGLU MoE composition with the interface of the reference's
+``flextrain/ops/full_moe.py`` (same function names, keyword arguments, slot
+fields and in-place conventions).
+
+What differs underneath: the per-expert Python loop (one GEMM call per expert,
+alternating two streams, after a device->host copy of the counts and a stream
+synchronisation: full_moe.py:144-148, :428-466, :545-626) is replaced by
+grouped launches that read the counts on the device.  ``secondary_stream`` is
+accepted and left idle: one grouped launch already fills the GPU.
+"""
+from __future__ import annotations
+
+from typing import Any, Callable, Mapping, MutableMapping
+
+import torch
+
+from .matmul_dispatcher import CublasLtDispatcher
+from .ops.grouped import flextrain_grouped_gemm_rows, flextrain_grouped_gemm_wgrad
+from .ops.moe import (
+    flextrain_fused_topk_softmax,
+    flextrain_load_balance_bwd,
+    flextrain_moe_gather,
+    flextrain_moe_router_gate_bwd,
+    flextrain_moe_scatter,
+    flextrain_moe_scatter_routing_weights,
+    flextrain_moe_sort,
+    flextrain_swiglu_moe_bwd,
+    flextrain_swiglu_moe_fwd,
+)
+
+_dispatcher = None
+
+
+def _get_dispatcher() -> CublasLtDispatcher:
+    """Created on first use so that importing this module touches no device
+    (the reference builds two dispatchers at import time,
+    flextrain/ops/_kernels/_matmul_dispatchers.py:3-4)."""
+    global _dispatcher
+    if _dispatcher is None:
+        _dispatcher = CublasLtDispatcher(round_multiple=32)
+    return _dispatcher
+
+
+def _device_counts(expert_counts_cpu, expert_counts_gpu):
+    """The grouped kernels read counts through a device pointer: device memory,
+    or pinned host memory (mapped into the device address space)."""
+    if expert_counts_gpu is not None:
+        return expert_counts_gpu
+    if expert_counts_cpu.is_cuda or expert_counts_cpu.is_pinned():
+        return expert_counts_cpu
+    return expert_counts_cpu.to("cuda", non_blocking=False)
+
+
+# ---------------------------------------------------------------------------
+# Phase ops (flextrain/ops/full_moe.py:77-174)
+# ---------------------------------------------------------------------------
+def route_topk_softmax(x, w_router, *, top_k, routing_mode, gate_logits_out, topk_ids_out, topk_weights_out):
+    """``gate_logits = x @ w_router`` then fused top-k softmax; all three output
+    buffers are written in place.  Returns ``(router_weights, topk_ids)``."""
+    s = torch.cuda.current_stream(x.device).cuda_stream
+    _get_dispatcher().matmul(s, A=x, B=w_router, D=gate_logits_out)
+    return flextrain_fused_topk_softmax(gate_logits_out, top_k=top_k, topk_ids_out=topk_ids_out,
+                                        topk_weights_out=topk_weights_out, mode=routing_mode)
+
+
+def dispatch_scatter(x, router_weights, topk_ids, *, num_experts, index_mapping, expert_counts_gpu,
+                     expert_counts_cpu, scattered_x_out, scattered_router_weights_out, sync=True):
+    """Sort (token, slot) pairs by expert, scatter ``x`` and the router weights
+    into sorted order, and fill both count buffers (the pinned host one is
+    written by the sort kernel itself).  ``sync=True`` keeps the reference
+    guarantee that the host counts are readable on return; the grouped expert
+    path does not need them and passes ``sync=False``."""
+    pinned = expert_counts_cpu if (expert_counts_cpu is not None and expert_counts_cpu.is_pinned()) else None
+    indices, _ = flextrain_moe_sort(topk_ids, num_experts=num_experts, indices=index_mapping,
+                                    expert_counts_gpu=expert_counts_gpu, expert_counts_pinned=pinned)
+    flextrain_moe_scatter(x, indices, out=scattered_x_out)
+    flextrain_moe_scatter_routing_weights(router_weights, indices, out=scattered_router_weights_out)
+    if expert_counts_cpu is not None and pinned is None:
+        expert_counts_cpu.copy_(expert_counts_gpu)  # pageable destination: synchronous copy
+    elif sync:
+        torch.cuda.current_stream(x.device).synchronize()
+    return indices, expert_counts_cpu
+
+
+def combine_gather(scattered_y, indices, *, router_weights, residual, out_tensor):
+    return flextrain_moe_gather(scattered_y, indices, residual=residual, weights=router_weights, out=out_tensor)
+
+
+# ---------------------------------------------------------------------------
+# Expert compute (flextrain/ops/full_moe.py:393-679)
+# ---------------------------------------------------------------------------
+def swiglu_expert_loop_fwd(scattered_x, x_preact_buf, w_up, w_down, expert_counts_cpu, *, primary_stream,
+                           secondary_stream=None, x_act_even=None, x_act_odd=None, expert_counts_gpu=None):
+    """For every expert e over its rows: ``x_preact = x_e @ w_up[e].T`` (saved),
+    ``act = silu(gate) * value``, ``scattered_x[rows] = act @ w_down[e].T``
+    (overwrites the input).  ``w_up (E, 2F, d)``, ``w_down (E, d, F)``."""
+    TK = scattered_x.shape[0]
+    F = w_down.shape[2]
+    counts = _device_counts(expert_counts_cpu, expert_counts_gpu)
+    with torch.cuda.stream(primary_stream):
+        pre = x_preact_buf[:TK]
+        flextrain_grouped_gemm_rows(scattered_x, w_up.transpose(1, 2), counts, pre)
+        if x_act_even is not None and x_act_even.shape[0] >= TK and x_act_even.shape[1] == F:
+            act = x_act_even[:TK]
+        else:
+            act = torch.empty((TK, F), dtype=scattered_x.dtype, device=scattered_x.device)
+        flextrain_swiglu_moe_fwd(pre, out=act)
+        flextrain_grouped_gemm_rows(act, w_down.transpose(1, 2), counts, scattered_x)
+
+
+def swiglu_expert_loop_bwd(scattered_upstream, scattered_x, x_preact_buf, srw, dprobs, w_up, w_down, grads,
+                           expert_counts_cpu, dx_up_up_grouped, dx_pre_grouped, *, expert_dim, primary_stream,
+                           secondary_stream=None, expert_counts_gpu=None):
+    """Backward of the expert block on expert-sorted rows (steps a-e of
+    flextrain/ops/full_moe.py:499-626): dgrad through ``w_down``, SwiGLU backward
+    (per-row router-weight gradient into ``dprobs``), ``g_down[e] +=``, dgrad
+    through ``w_up`` into ``dx_pre_grouped``, ``g_up[e] +=``.  A gradient
+    accumulator missing from ``grads`` (or None) is skipped."""
+    TK = scattered_upstream.shape[0]
+    counts = _device_counts(expert_counts_cpu, expert_counts_gpu)
+    with torch.cuda.stream(primary_stream):
+        dx_act = torch.empty((TK, expert_dim), dtype=scattered_upstream.dtype, device=scattered_upstream.device)
+        fwd_act = torch.empty_like(dx_act)
+        flextrain_grouped_gemm_rows(scattered_upstream, w_down, counts, dx_act)                        # (a)
+        flextrain_swiglu_moe_bwd(dx_act, x_preact_buf[:TK], srw[:TK], dx=dx_up_up_grouped[:TK], dw=dprobs[:TK],
+                                 fwd_act=fwd_act)                                                       # (b)
+        if grads.get("g_down") is not None:
+            flextrain_grouped_gemm_wgrad(scattered_upstream, fwd_act, grads["g_down"], counts)          # (c)
+        flextrain_grouped_gemm_rows(dx_up_up_grouped[:TK], w_up, counts, dx_pre_grouped[:TK])           # (d)
+        if grads.get("g_up") is not None:
+            flextrain_grouped_gemm_wgrad(dx_up_up_grouped[:TK], scattered_x, grads["g_up"], counts)     # (e)
+
+
+def swiglu_expert_loop_recompute_x_up(scattered_x, x_preact_buf, w_up, expert_counts_cpu, *, primary_stream,
+                                      secondary_stream=None, expert_counts_gpu=None):
+    """Refill ``x_preact_buf`` from the saved scattered input (up-projection only)."""
+    counts = _device_counts(expert_counts_cpu, expert_counts_gpu)
+    with torch.cuda.stream(primary_stream):
+        flextrain_grouped_gemm_rows(scattered_x, w_up.transpose(1, 2), counts, x_preact_buf[:scattered_x.shape[0]])
+
+
+# ---------------------------------------------------------------------------
+# End-to-end ops (flextrain/ops/full_moe.py:177-390)
+# ---------------------------------------------------------------------------
+def routed_swiglu_moe_fwd(ffn_norm_output, weights: Mapping[str, torch.Tensor], *, out_tensor, residual, slot: Any,
+                          chunk_extra: MutableMapping[str, Any], layer_id: int, top_k: int, num_experts: int,
+                          routing_mode: str, primary_stream, secondary_stream,
+                          scratch_fn: Callable[[tuple, torch.dtype], torch.Tensor], expert_compute) -> None:
+    """Router, then the backend's scatter + expert MLP + gather.  Fills the
+    slot's router fields and writes the residual-added output into ``out_tensor``."""
+    router_weights, topk_ids = route_topk_softmax(
+        ffn_norm_output, weights["w_router"], top_k=top_k, routing_mode=routing_mode,
+        gate_logits_out=slot.x_router, topk_ids_out=slot.chosen_experts, topk_weights_out=slot.router_weights)
+    expert_compute.fwd(
+        ffn_norm_output, router_weights, topk_ids, weights, out=out_tensor,
+        residual=residual if expert_compute.supports_residual_in_gather else None, slot=slot,
+        chunk_extra=chunk_extra, layer_id=layer_id, primary_stream=primary_stream,
+        secondary_stream=secondary_stream, scratch_fn=scratch_fn)
+    if not expert_compute.supports_residual_in_gather and residual is not None:
+        out_tensor.add_(residual.view(-1, ffn_norm_output.shape[-1]))
+
+
+def routed_swiglu_moe_bwd(dy_resid, weights, grads, slot, chunk_extra, layer_id, *, ffn_norm_output, top_k,
+                          num_experts, routing_mode, load_balance_coef, total_tokens_per_step, primary_stream,
+                          secondary_stream, scratch_fn, expert_compute, scattered_x_recompute=None,
+                          lora_capture=None):
+    """Returns the gradient at the FFN-norm output.  Backend bwd, router-gate
+    bwd, optional load-balance gradient, then ``dx += dlogits @ w_router.T`` and
+    ``g_router += x.T @ dlogits``."""
+    num_tokens, d_model = dy_resid.shape
+    stream_ptr = primary_stream.cuda_stream
+    kwargs = dict(slot=slot, chunk_extra=chunk_extra, layer_id=layer_id, primary_stream=primary_stream,
+                  secondary_stream=secondary_stream, scratch_fn=scratch_fn,
+                  recompute_handoff=scattered_x_recompute)
+    if lora_capture is not None:
+        kwargs["lora_capture"] = lora_capture
+    ffn_norm_upstream = expert_compute.bwd(dy_resid, ffn_norm_output, weights, grads, **kwargs)
+    dprobs = slot.aux.pop("moe_dprobs")
+    dlogits = torch.zeros((num_tokens, num_experts), dtype=dy_resid.dtype, device=dy_resid.device)
+    flextrain_moe_router_gate_bwd(slot.router_weights, dprobs, slot.index_mapping, slot.chosen_experts,
+                                  dlogits=dlogits, mode=routing_mode, logits=slot.x_router)
+    if load_balance_coef > 0.0 and total_tokens_per_step is not None:
+        flextrain_load_balance_bwd(logits=slot.x_router, expert_counts=expert_compute.expert_counts_gpu(slot),
+                                   num_experts=num_experts, alpha=load_balance_coef,
+                                   tokens_per_step=total_tokens_per_step, top_k=top_k, dlogits=dlogits)
+    disp = _get_dispatcher()
+    disp.matmul(stream_ptr, A=dlogits, B=weights["w_router"].T, C=ffn_norm_upstream, D=ffn_norm_upstream,
+                beta=1.0, alpha=1.0)
+    if grads.get("g_router") is not None:
+        disp.matmul(stream_ptr, A=ffn_norm_output.T, B=dlogits, C=grads["g_router"], D=grads["g_router"],
+                    beta=1.0, alpha=1.0)
+    return ffn_norm_upstream
+
+
+def routed_swiglu_moe_recompute_x_up(ffn_norm_output, weights, slot, chunk_extra, layer_id, *, primary_stream,
+                                     secondary_stream, scratch_fn, expert_compute):
+    return expert_compute.fwd_recompute(ffn_norm_output, weights, slot=slot, chunk_extra=chunk_extra,
+                                        layer_id=layer_id, primary_stream=primary_stream,
+                                        secondary_stream=secondary_stream, scratch_fn=scratch_fn)
+
+
+__all__ = (
+    "routed_swiglu_moe_fwd",
+    "routed_swiglu_moe_bwd",
+    "routed_swiglu_moe_recompute_x_up",
+    "route_topk_softmax",
+    "dispatch_scatter",
+    "combine_gather",
+    "swiglu_expert_loop_fwd",
+    "swiglu_expert_loop_bwd",
+    "swiglu_expert_loop_recompute_x_up",
+)

@@ -1,0 +1,160 @@
+"""GEMM dispatcher with the interface of the reference's ``matmul_dispatcher``
+package (helpers/matmul_dispatcher/matmul_dispatcher/__init__.py:63-276):
+``D = alpha * A @ B + beta * C`` on strided row-major / column-major 2-D
+tensors, fp32 accumulation, explicit stream pointer.
+
+``CublasLtDispatcher`` is kept as the class name callers import; it drives the
+hand-written MFMA GEMM of libflexhip.so through ``dispatch_matmul``.  No
+workspace is allocated (the kernel needs none), and nothing touches the GPU at
+import or construction time.
+"""
+from __future__ import annotations
+
+import ctypes
+import time
+
+import torch
+
+from ._lib import lib
+
+_dtype_to_enum = {torch.float16: 1, torch.bfloat16: 2, torch.float32: 0}
+
+
+def _get_layout(t):
+    """``(data_ptr, leading_dim, trans_flag)``: unit column stride -> row-major
+    (trans 0, ld = row stride); unit row stride -> column-major (trans 1,
+    ld = column stride).  helpers/matmul_dispatcher/matmul_dispatcher/__init__.py:63-90."""
+    if t.dim() != 2:
+        raise ValueError("Only 2D tensors supported for matmul dispatcher.")
+    stride_row, stride_col = t.stride()
+    if stride_col == 1:
+        return t.data_ptr(), stride_row, 0
+    if stride_row == 1:
+        return t.data_ptr(), stride_col, 1
+    raise ValueError(
+        f"Tensor memory layout not supported (Strides: {t.stride()}). "
+        "Must be Row-Major (stride[:,-1]==1) or Col-Major (stride[:,0]==1).")
+
+
+def tensor_layout(t):
+    """Return ``(data_ptr, leading_dim, trans_flag)`` for a 2-D tensor."""
+    return _get_layout(t)
+
+
+def dtype_enum(dtype):
+    """torch dtype -> 0 fp32 / 1 fp16 / 2 bf16."""
+    try:
+        return _dtype_to_enum[dtype]
+    except KeyError:
+        raise ValueError(f"unsupported dtype {dtype} for matmul_fast") from None
+
+
+def matmul_fast(ctx_int, stream, M, N, K, ptr_A, lda, trans_a, ptr_B, ldb, trans_b, ptr_C, ldc, ptr_D, ldd,
+                ws_ptr, ws_bytes, a_dt, b_dt, c_dt, d_dt, compute_dt, alpha, beta):
+    """Raw 24-argument entry with the argument order of the reference's
+    ``matmul_fast`` (helpers/matmul_dispatcher/src/dispatch_pyext.cpp:37-140).
+    Raises ``RuntimeError`` when ``dispatch_matmul`` reports failure."""
+    rc = lib().dispatch_matmul(ctx_int, stream, M, N, K, ptr_A, lda, ptr_B, ldb, ptr_C, ldc, ptr_D, ldd,
+                               ws_ptr, ws_bytes, a_dt, b_dt, c_dt, d_dt, compute_dt, alpha, beta,
+                               trans_a, trans_b)
+    if rc != 0:
+        raise RuntimeError(f"dispatch_matmul failed (rc={rc})")
+
+
+class CublasLtDispatcher:
+    """Same constructor and methods as the reference class of this name
+    (helpers/matmul_dispatcher/matmul_dispatcher/__init__.py:125-276)."""
+
+    def __init__(self, round_multiple=32, max_algos=5):
+        self.round_multiple = round_multiple
+        self.max_algos = max_algos
+        self._lib = lib()
+        self.ctx = self._lib.create_dispatcher(round_multiple, max_algos)
+        self.workspace_size = 0
+        self.workspace = None
+        self.ws_ptr = 0
+        self.fp16 = torch.float16
+        self.bf16 = torch.bfloat16
+        self.total_python_ns = 0
+        self._ctx_int = int(self.ctx) if self.ctx is not None else 0
+
+    def __del__(self):
+        if getattr(self, "ctx", None):
+            self._lib.destroy_dispatcher(self.ctx)
+            self.ctx = None
+
+    def get_stats(self):
+        stats = (ctypes.c_uint64 * 7)()
+        self._lib.get_stats(self.ctx, stats)
+        calls = stats[1]
+        if calls == 0:
+            return {"matmuls_called": 0, "algos_saved": 0, "algo_hits": 0, "avg_wrapper_overhead_us": 0,
+                    "avg_cpp_total_us": 0, "breakdown": {"driver_submit_us": 0, "cpp_hash_logic_us": 0}}
+        total_cpp_ns, total_driver_ns = stats[3], stats[6]
+        return {
+            "matmuls_called": calls,
+            "algos_saved": stats[0],
+            "algo_hits": stats[2],
+            "avg_wrapper_overhead_us": (self.total_python_ns / calls / 1000.0) - (total_cpp_ns / calls / 1000.0),
+            "avg_cpp_total_us": total_cpp_ns / calls / 1000.0,
+            "breakdown": {"driver_submit_us": total_driver_ns / calls / 1000.0,
+                          "cpp_hash_logic_us": (total_cpp_ns - total_driver_ns) / calls / 1000.0},
+        }
+
+    def matmul(self, stream_ptr, A, B, C=None, D=None, alpha=1.0, beta=0.0):
+        """``D = alpha * A @ B + beta * C``; allocates ``D`` when it is None."""
+        t0 = time.perf_counter_ns()
+        ptr_A, ld_A, trans_a = _get_layout(A)
+        ptr_B, ld_B, trans_b = _get_layout(B)
+        M, K = A.shape
+        K_B, N = B.shape
+        if K != K_B:
+            raise ValueError(f"Shape Mismatch: A is {A.shape}, B is {B.shape}. Inner dims {K} vs {K_B} must match.")
+        if D is None:
+            D = torch.empty((M, N), dtype=A.dtype, device=A.device)
+        ptr_D, ld_D, trans_d = _get_layout(D)
+        if trans_d != 0:
+            raise ValueError("Output tensor D must be Row-Major for this dispatcher.")
+        if C is not None:
+            ptr_C, ld_C, trans_c = _get_layout(C)
+            if trans_c != 0:
+                raise ValueError("Bias/Add tensor C must be Row-Major.")
+        else:
+            ptr_C, ld_C = 0, N
+        if M == 0 or N == 0 or K == 0:
+            raise ValueError(f"All dimensions must be non-zero. Got M={M}, N={N}, K={K}")
+        dt = 1 if A.dtype == self.fp16 else (2 if A.dtype == self.bf16 else 0)
+        d_dt = _dtype_to_enum.get(D.dtype, dt)
+        ret = self._lib.dispatch_matmul(self.ctx, stream_ptr, M, N, K, ptr_A, ld_A, ptr_B, ld_B, ptr_C, ld_C,
+                                        ptr_D, ld_D, self.ws_ptr, self.workspace_size, dt, dt, d_dt, d_dt, 0,
+                                        alpha, beta, trans_a, trans_b)
+        if ret != 0:
+            raise RuntimeError("Failed to dispatch matmul")
+        self.total_python_ns += time.perf_counter_ns() - t0
+        return D
+
+    def matmul_fast(self, stream_ptr, A, B, C=None, D=None, alpha=1.0, beta=0.0):
+        """Hot-path variant: no validation, no allocation (``D`` required), no
+        wrapper timing.  Bit-identical results to :meth:`matmul`."""
+        a_stride = A.stride()
+        if a_stride[1] == 1:
+            ptr_A, ld_A, trans_a = A.data_ptr(), a_stride[0], 0
+        else:
+            ptr_A, ld_A, trans_a = A.data_ptr(), a_stride[1], 1
+        b_stride = B.stride()
+        if b_stride[1] == 1:
+            ptr_B, ld_B, trans_b = B.data_ptr(), b_stride[0], 0
+        else:
+            ptr_B, ld_B, trans_b = B.data_ptr(), b_stride[1], 1
+        ptr_D, ld_D = D.data_ptr(), D.stride(0)
+        if C is None:
+            ptr_C, ld_C = 0, ld_D
+        else:
+            ptr_C, ld_C = C.data_ptr(), C.stride(0)
+        M, K = A.shape
+        _, N = B.shape
+        dt = _dtype_to_enum[A.dtype]
+        d_dt = _dtype_to_enum[D.dtype]
+        matmul_fast(self._ctx_int, stream_ptr, M, N, K, ptr_A, ld_A, trans_a, ptr_B, ld_B, trans_b, ptr_C, ld_C,
+                    ptr_D, ld_D, self.ws_ptr, self.workspace_size, dt, dt, d_dt, d_dt, 0, alpha, beta)
+        return D

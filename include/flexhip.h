@@ -184,6 +184,50 @@ int fx_swiglu_moe_bwd(void* dx, void* dw, int dw_dt, const void* dout, const voi
                       void* fwd_act, int64_t rows, int F, int64_t dx_row_stride, int64_t dout_row_stride,
                       int64_t x_row_stride, int64_t act_row_stride, int dt, int prescaled, hipStream_t stream);
 
+/* ---- Expert-grouped GEMMs -------------------------------------------------- */
+
+/* Scratch bytes for the two grouped GEMM entry points (row offsets + tile list). */
+size_t fx_grouped_ws_bytes(int E, int64_t total_rows);
+
+/* The per-expert GEMMs of swiglu_expert_loop_fwd / _bwd / _recompute_x_up
+ * (flextrain/ops/full_moe.py:428-466, :589-601, :613-616, :661-676) as one launch:
+ *   D_e[c_e, N] = alpha * A_e[c_e, K] * op(B[e]) + beta * C_e
+ * for every expert e, rows [off_e, off_e + c_e) of the expert-sorted buffers A, C, D.
+ * counts: E int32 readable by the device (device memory or pinned host memory).
+ * B[e] = B + e * b_expert_stride; trans_b = 1: B[e] stored (N,K) (x @ w.T);
+ * trans_b = 0: B[e] stored (K,N).  C may be NULL.  dt: fp16 or bf16. */
+int fx_grouped_gemm_rows(const void* A, int64_t lda, const void* B, int64_t ldb, int64_t b_expert_stride,
+                         int trans_b, const void* C, int64_t ldc, void* D, int64_t ldd, const int32_t* counts,
+                         int E, int64_t total_rows, int N, int K, float alpha, float beta, int dt, void* ws,
+                         size_t ws_bytes, hipStream_t stream);
+
+/* The per-expert weight-gradient GEMMs (flextrain/ops/full_moe.py:602-611, :617-626):
+ *   G[e][M, N] = alpha * A_e[c_e, M]^T * B_e[c_e, N] + beta * G[e],  G[e] = G + e * g_expert_stride.
+ * g_dt may be fp32 for bf16 inputs. */
+int fx_grouped_gemm_wgrad(const void* A, int64_t lda, const void* B, int64_t ldb, void* G, int64_t ldg,
+                          int64_t g_expert_stride, int g_dt, const int32_t* counts, int E, int64_t total_rows,
+                          int M, int N, float alpha, float beta, int dt, void* ws, size_t ws_bytes,
+                          hipStream_t stream);
+
+/* ---- GEMM dispatcher (verbatim ABI of the reference helper) --------------- */
+
+/* helpers/matmul_dispatcher/src/dispatch.h:12-35.  D = alpha*op(A)*op(B) + beta*C,
+ * row-major storage, fp32 accumulation.  trans_a = 0: A is (M,K) with row
+ * stride lda; trans_a = 1: A is stored (K,M) with row stride lda.  trans_b = 0:
+ * B is (K,N) with row stride ldb; trans_b = 1: B is stored (N,K).  C may be 0
+ * (treated as beta = 0) and may alias D.  M, N or K == 0 returns 0 without
+ * doing anything.  The workspace arguments are accepted and unused.  A context
+ * is not thread-safe; use one per stream, as the reference does. */
+typedef struct DispatchContext DispatchContext;
+DispatchContext* create_dispatcher(int round_multiple, int max_algos);
+void destroy_dispatcher(DispatchContext* ctx);
+/* out_stats[7] = {algos_saved, calls, hits, total_ns, hash_ns, lookup_ns, driver_ns}. */
+void get_stats(DispatchContext* ctx, uint64_t* out_stats);
+int dispatch_matmul(DispatchContext* ctx, intptr_t stream_ptr, int M, int N, int K, intptr_t ptr_A, int lda,
+                    intptr_t ptr_B, int ldb, intptr_t ptr_C, int ldc, intptr_t ptr_D, int ldd,
+                    intptr_t ptr_workspace, size_t workspace_bytes, int a_dt, int b_dt, int c_dt, int d_dt,
+                    int compute_dt, float alpha, float beta, int trans_a, int trans_b);
+
 #ifdef __cplusplus
 }
 #endif

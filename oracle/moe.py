@@ -199,3 +199,72 @@ def grouped_expert_bwd(dyg, xg, pre, wsorted, counts, w_up, w_down, g_up=None, g
         dx[a:b] = (dx_up.float() @ w_up[e].float()).to(xg.dtype)
         gu[e] += dx_up.float().t() @ xg[a:b].float()
     return dx, dprobs, gu, gd
+
+
+# ------------------------------------------------------------ whole block
+def routed_block_fwd_bwd(x, logits, w_router, w_up, w_down, residual, dy, top_k, mode="topk_then_softmax",
+                         load_balance_coef=0.0, tokens_per_step=None, experts=None):
+    """The routed-SwiGLU block of flextrain/ops/full_moe.py:177-362 from given router
+    logits (so that routing does not depend on GEMM rounding): forward output, and
+    backward dx (including the router path), g_up, g_down, g_router.
+
+    ``experts``: optional subset of expert ids to evaluate the expert MLP for (rows
+    of other experts contribute zero) — used to bound CPU time at full size.
+    Returns a dict of tensors."""
+    T, d = x.shape
+    E = w_up.shape[0]
+    w, ids = topk_softmax(logits, top_k, mode=mode)
+    mapping, counts = moe_sort(ids, E)
+    if experts is not None:
+        keep = torch.zeros(E, dtype=torch.bool)
+        keep[list(experts)] = True
+        counts_eval = torch.where(keep, counts, torch.zeros_like(counts))
+    xg = moe_scatter(x, mapping)
+    wsorted = moe_scatter_routing_weights(w, mapping)
+    off = expert_offsets(counts)
+
+    def run(fn_rows):
+        # evaluate per expert on its true row range, skipping unselected experts
+        for e in range(E):
+            a, b = int(off[e]), int(off[e + 1])
+            if a == b or (experts is not None and e not in experts):
+                continue
+            fn_rows(e, a, b)
+
+    TK = T * top_k
+    F2 = w_up.shape[1]
+    pre = torch.zeros(TK, F2, dtype=x.dtype)
+    y = torch.zeros(TK, d, dtype=x.dtype)
+
+    def fwd_rows(e, a, b):
+        pre[a:b] = (xg[a:b].float() @ w_up[e].float().t()).to(x.dtype)
+        act = swiglu_moe_fwd(pre[a:b])
+        y[a:b] = (act.float() @ w_down[e].float().t()).to(x.dtype)
+
+    run(fwd_rows)
+    out = moe_gather(y, mapping, w, residual)
+
+    dyg = moe_scatter(dy, mapping)
+    dxg = torch.zeros(TK, d, dtype=x.dtype)
+    dprobs = torch.zeros(TK, dtype=torch.float32)
+    g_up = torch.zeros(E, F2, d)
+    g_down = torch.zeros(E, d, F2 // 2)
+
+    def bwd_rows(e, a, b):
+        dact = (dyg[a:b].float() @ w_down[e].float()).to(x.dtype)
+        dx_up, dw, act_w = swiglu_moe_bwd(dact, pre[a:b], wsorted[a:b])
+        dprobs[a:b] = dw
+        g_down[e] = dyg[a:b].float().t() @ act_w.float()
+        dxg[a:b] = (dx_up.float() @ w_up[e].float()).to(x.dtype)
+        g_up[e] = dx_up.float().t() @ xg[a:b].float()
+
+    run(bwd_rows)
+    dx = moe_gather(dxg, mapping)
+    dprobs_b = dprobs.to(x.dtype)                      # the backend's dprobs buffer is in compute dtype
+    dlogits = router_gate_bwd(w, dprobs_b, mapping, ids, E, mode=mode, logits=logits)
+    if load_balance_coef > 0.0 and tokens_per_step is not None:
+        dlogits = load_balance_bwd(logits, counts, top_k, load_balance_coef, tokens_per_step, dlogits)
+    dx_total = (dx.float() + dlogits.float() @ w_router.float().t()).to(x.dtype)
+    g_router = x.float().t() @ dlogits.float()
+    return dict(out=out, dx=dx_total, dx_experts=dx, g_up=g_up, g_down=g_down, g_router=g_router, ids=ids,
+                weights=w, mapping=mapping, counts=counts, pre=pre, dlogits=dlogits)
