@@ -55,7 +55,7 @@ FX_DEV float row_sum(float v, float* red, int tid) {
 // ---------------------------------------------------------------------------
 template <typename T, int LPR, int MAXV, int THREADS, bool SAVED_RSTD>
 __global__ __launch_bounds__(THREADS) void rmsnorm_fwd_kernel(
-    const T* __restrict__ X, const void* __restrict__ W, int w_dt, T* __restrict__ Y,
+    const T* X, const void* __restrict__ W, int w_dt, T* Y /* may alias X */,
     float* __restrict__ RSTD, int64_t rows, int ncols, float eps) {
     constexpr int G = THREADS / LPR;  // rows per workgroup
     __shared__ float red[THREADS / 64];
@@ -111,7 +111,7 @@ __global__ __launch_bounds__(THREADS) void rmsnorm_fwd_kernel(
 // Any-shape fallback: one workgroup per row, two passes over the row.
 template <typename T, bool SAVED_RSTD>
 __global__ __launch_bounds__(256) void rmsnorm_fwd_generic_kernel(
-    const T* __restrict__ X, const void* __restrict__ W, int w_dt, T* __restrict__ Y,
+    const T* X, const void* __restrict__ W, int w_dt, T* Y /* may alias X */,
     float* __restrict__ RSTD, int64_t rows, int ncols, float eps) {
     __shared__ float red[4];
     __shared__ float s_rstd;

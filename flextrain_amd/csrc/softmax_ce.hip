@@ -1,0 +1,241 @@
+// Row softmax, cross-entropy from probabilities, and the fused
+// logits -> (loss, dZ) kernel of the LM head, gfx950.
+//
+// Reference semantics:
+//   flextrain/ops/_kernels/softmax.py:13-108        online softmax with temperature; probabilities
+//                                                   rounded to the output dtype; first-occurrence
+//                                                   argmax (int64) and max probability 1/l (fp32)
+//   flextrain/ops/_kernels/cross_entropy.py:14-57   valid = 0 <= label < V; loss = min(-log p[label],
+//                                                   max_loss); p[label] -= 1 in place
+//   flextrain/nn/loss.py:248-316                    rows whose label is the ignore index (or whose
+//                                                   loss_mask is false) get loss 0 and a zero dZ row
+// The fused kernel does all of the above in two sweeps over a row of logits and
+// takes the loss from the fp32 log-sum-exp, lse - logit[label], instead of from
+// probabilities already rounded to bf16.
+//
+// One workgroup of 1024 lanes owns a row; a lane keeps an online (max, sum)
+// pair over its 16-byte packs, pairs are merged through wave shuffles and LDS.
+#include "common.h"
+#include "flexhip.h"
+
+namespace fx {
+
+constexpr int SM_THREADS = 1024;
+constexpr float NEG_INF_F = -__builtin_huge_valf();
+
+struct RowStat {
+    float m, l, best;
+    int idx;
+};
+
+FX_DEV void stat_add(RowStat& s, float x, int i) {
+    if (x > s.best) { s.best = x; s.idx = i; }        // strict: the first maximum wins
+    if (x > s.m) {
+        s.l = s.l * __expf(s.m - x) + 1.0f;
+        s.m = x;
+    } else if (x > NEG_INF_F) {   // a -inf element adds nothing (and -inf - -inf is NaN)
+        s.l += __expf(x - s.m);
+    }
+}
+
+FX_DEV void stat_merge(RowStat& a, float m, float l, float best, int idx) {
+    if (best > a.best || (best == a.best && idx < a.idx)) { a.best = best; a.idx = idx; }
+    const float nm = fmaxf(a.m, m);
+    if (nm == NEG_INF_F) { a.l = 0.f; a.m = nm; return; }
+    a.l = a.l * __expf(a.m - nm) + l * __expf(m - nm);
+    a.m = nm;
+}
+
+// All lanes of the workgroup return the row's merged statistics.
+FX_DEV RowStat block_stat(RowStat s, float* sm_f, int* sm_i) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float m = __shfl_xor(s.m, off, 64), l = __shfl_xor(s.l, off, 64), b = __shfl_xor(s.best, off, 64);
+        const int i = __shfl_xor(s.idx, off, 64);
+        stat_merge(s, m, l, b, i);
+    }
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    constexpr int NW = SM_THREADS / 64;
+    __syncthreads();
+    if (lane == 0) { sm_f[wave] = s.m; sm_f[NW + wave] = s.l; sm_f[2 * NW + wave] = s.best; sm_i[wave] = s.idx; }
+    __syncthreads();
+    RowStat r{sm_f[0], sm_f[NW], sm_f[2 * NW], sm_i[0]};
+    for (int w = 1; w < NW; ++w) stat_merge(r, sm_f[w], sm_f[NW + w], sm_f[2 * NW + w], sm_i[w]);
+    return r;
+}
+
+template <typename T>
+FX_DEV RowStat row_sweep(const T* __restrict__ x, int V, float inv_temp, bool vec) {
+    RowStat s{NEG_INF_F, 0.f, NEG_INF_F, 0x7fffffff};
+    if (vec) {
+        for (int c = threadIdx.x * 8; c < V; c += SM_THREADS * 8) {
+            float v[8];
+            load_f32<T, 8>(x + c, v);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) stat_add(s, v[j] * inv_temp, c + j);
+        }
+    } else {
+        for (int c = threadIdx.x; c < V; c += SM_THREADS) stat_add(s, (float)x[c] * inv_temp, c);
+    }
+    return s;
+}
+
+template <typename TI, typename TO>
+__global__ __launch_bounds__(SM_THREADS) void softmax_kernel(
+    const TI* __restrict__ X, TO* __restrict__ OUT, int64_t* __restrict__ MAX_IDX, float* __restrict__ MAX_VAL,
+    int V, int64_t in_stride, int64_t out_stride, float inv_temp, bool vec) {
+    __shared__ float sm_f[3 * SM_THREADS / 64];
+    __shared__ int sm_i[SM_THREADS / 64];
+    const int64_t row = blockIdx.x;
+    const TI* x = X + row * in_stride;
+    TO* o = OUT + row * out_stride;
+    const RowStat st = block_stat(row_sweep<TI>(x, V, inv_temp, vec), sm_f, sm_i);
+    const float inv_l = 1.0f / st.l;
+    if (threadIdx.x == 0) {
+        if (MAX_IDX) MAX_IDX[row] = st.idx;
+        if (MAX_VAL) MAX_VAL[row] = inv_l;
+    }
+    if (vec) {
+        for (int c = threadIdx.x * 8; c < V; c += SM_THREADS * 8) {
+            float v[8];
+            load_f32<TI, 8>(x + c, v);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = __expf(v[j] * inv_temp - st.m) * inv_l;
+            store_f32<TO, 8>(o + c, v);
+        }
+    } else {
+        for (int c = threadIdx.x; c < V; c += SM_THREADS) o[c] = (TO)(__expf((float)x[c] * inv_temp - st.m) * inv_l);
+    }
+}
+
+// Probabilities in, dZ out (in place), one lane per row.
+template <typename T, typename TL>
+__global__ __launch_bounds__(256) void cross_entropy_kernel(T* __restrict__ P, const TL* __restrict__ LABELS,
+                                                            float* __restrict__ LOSS, float* __restrict__ VALID,
+                                                            int64_t rows, int V, int64_t stride_t, int64_t stride_v,
+                                                            float max_loss) {
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= rows) return;
+    const int64_t label = (int64_t)LABELS[t];
+    const bool valid = label >= 0 && label < V;
+    VALID[t] = valid ? 1.0f : 0.0f;
+    float loss = 0.f;
+    if (valid) {
+        T* p = P + t * stride_t + label * stride_v;
+        const float pc = (float)*p;
+        loss = fminf(-logf(pc), max_loss);
+        *p = (T)(pc - 1.0f);
+    }
+    LOSS[t] = loss;
+}
+
+// Logits in, dZ out (in place or to DZ), fp32 loss from the log-sum-exp.
+//   keep  = label != ignore_index  &&  (MASK == null || MASK[t])
+//   valid = 0 <= label < V
+//   loss  = keep && valid ? min(lse - x[label], max_loss) : 0
+//   dZ    = keep ? softmax(x) - (valid ? onehot(label) : 0) : 0
+template <typename T, typename TL>
+__global__ __launch_bounds__(SM_THREADS) void softmax_ce_kernel(
+    const T* X, T* DZ /* may alias X */, const TL* __restrict__ LABELS, const uint8_t* __restrict__ MASK,
+    float* __restrict__ LOSS, int64_t* __restrict__ MAX_IDX, float* __restrict__ MAX_VAL, int V, int64_t in_stride,
+    int64_t out_stride, int64_t ignore_index, float max_loss, bool vec) {
+    __shared__ float sm_f[3 * SM_THREADS / 64];
+    __shared__ int sm_i[SM_THREADS / 64];
+    const int64_t row = blockIdx.x;
+    const T* x = X + row * in_stride;
+    T* o = DZ + row * out_stride;
+    const int64_t label = (int64_t)LABELS[row];
+    const bool keep = label != ignore_index && (MASK == nullptr || MASK[row] != 0);
+    const bool valid = label >= 0 && label < V;
+    const RowStat st = block_stat(row_sweep<T>(x, V, 1.0f, vec), sm_f, sm_i);
+    const float inv_l = 1.0f / st.l;
+    if (threadIdx.x == 0) {
+        if (MAX_IDX) MAX_IDX[row] = st.idx;
+        if (MAX_VAL) MAX_VAL[row] = inv_l;
+        float loss = 0.f;
+        if (keep && valid) loss = fminf((st.m + logf(st.l)) - (float)x[label], max_loss);
+        LOSS[row] = loss;
+    }
+    __syncthreads();  // x[label] is read before any lane overwrites the row in place
+    const int hot = (keep && valid) ? (int)label : -1;
+    if (vec) {
+        for (int c = threadIdx.x * 8; c < V; c += SM_THREADS * 8) {
+            float v[8];
+            if (keep) {
+                load_f32<T, 8>(x + c, v);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    v[j] = __expf(v[j] - st.m) * inv_l;
+                    if (c + j == hot) v[j] -= 1.0f;
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) v[j] = 0.f;
+            }
+            store_f32<T, 8>(o + c, v);
+        }
+    } else {
+        for (int c = threadIdx.x; c < V; c += SM_THREADS) {
+            float v = 0.f;
+            if (keep) {
+                v = __expf((float)x[c] - st.m) * inv_l;
+                if (c == hot) v -= 1.0f;
+            }
+            o[c] = (T)v;
+        }
+    }
+}
+
+}  // namespace fx
+
+using namespace fx;
+
+extern "C" int fx_softmax(const void* x, void* out, int64_t* max_idx_out, float* max_val_out, int64_t rows, int V,
+                          int64_t in_row_stride, int64_t out_row_stride, float temperature, int in_dt, int out_dt,
+                          hipStream_t stream) {
+    if (rows < 0 || V <= 0) FX_FAIL("fx_softmax: bad shape");
+    if (!(temperature > 0.f)) FX_FAIL("fx_softmax: temperature must be positive");
+    if (rows == 0) return 0;
+    if (!x || !out) FX_FAIL("fx_softmax: null pointer");
+    const bool vec = (V % 8 == 0) && (in_row_stride % 8 == 0) && (out_row_stride % 8 == 0) && aligned16(x) && aligned16(out);
+    FX_DISPATCH_DTYPE(in_dt, TI,
+        FX_DISPATCH_DTYPE(out_dt, TO,
+            softmax_kernel<TI, TO><<<(unsigned)rows, SM_THREADS, 0, stream>>>(
+                reinterpret_cast<const TI*>(x), reinterpret_cast<TO*>(out), max_idx_out, max_val_out, V, in_row_stride,
+                out_row_stride, 1.0f / temperature, vec)));
+    FX_CHECK_LAUNCH("fx_softmax");
+    return 0;
+}
+
+extern "C" int fx_cross_entropy(void* probs, const void* labels, int labels_are_int64, float* loss_out,
+                                float* valid_out, int64_t rows, int V, int64_t stride_t, int64_t stride_v,
+                                float max_loss, int dt, hipStream_t stream) {
+    if (rows < 0 || V <= 0) FX_FAIL("fx_cross_entropy: bad shape");
+    if (rows == 0) return 0;
+    if (!probs || !labels || !loss_out || !valid_out) FX_FAIL("fx_cross_entropy: null pointer");
+    const unsigned grid = (unsigned)((rows + 255) / 256);
+    FX_DISPATCH_DTYPE(dt, TT,
+        if (labels_are_int64)
+            cross_entropy_kernel<TT, int64_t><<<grid, 256, 0, stream>>>(reinterpret_cast<TT*>(probs), reinterpret_cast<const int64_t*>(labels), loss_out, valid_out, rows, V, stride_t, stride_v, max_loss);
+        else
+            cross_entropy_kernel<TT, int32_t><<<grid, 256, 0, stream>>>(reinterpret_cast<TT*>(probs), reinterpret_cast<const int32_t*>(labels), loss_out, valid_out, rows, V, stride_t, stride_v, max_loss));
+    FX_CHECK_LAUNCH("fx_cross_entropy");
+    return 0;
+}
+
+extern "C" int fx_softmax_ce(const void* logits, void* dz_out, const void* labels, int labels_are_int64,
+                             const uint8_t* loss_mask, float* loss_out, int64_t* max_idx_out, float* max_val_out,
+                             int64_t rows, int V, int64_t in_row_stride, int64_t out_row_stride, int64_t ignore_index,
+                             float max_loss, int dt, hipStream_t stream) {
+    if (rows < 0 || V <= 0) FX_FAIL("fx_softmax_ce: bad shape");
+    if (rows == 0) return 0;
+    if (!logits || !dz_out || !labels || !loss_out) FX_FAIL("fx_softmax_ce: null pointer");
+    const bool vec = (V % 8 == 0) && (in_row_stride % 8 == 0) && (out_row_stride % 8 == 0) && aligned16(logits) && aligned16(dz_out);
+    FX_DISPATCH_DTYPE(dt, TT,
+        if (labels_are_int64)
+            softmax_ce_kernel<TT, int64_t><<<(unsigned)rows, SM_THREADS, 0, stream>>>(reinterpret_cast<const TT*>(logits), reinterpret_cast<TT*>(dz_out), reinterpret_cast<const int64_t*>(labels), loss_mask, loss_out, max_idx_out, max_val_out, V, in_row_stride, out_row_stride, ignore_index, max_loss, vec);
+        else
+            softmax_ce_kernel<TT, int32_t><<<(unsigned)rows, SM_THREADS, 0, stream>>>(reinterpret_cast<const TT*>(logits), reinterpret_cast<TT*>(dz_out), reinterpret_cast<const int32_t*>(labels), loss_mask, loss_out, max_idx_out, max_val_out, V, in_row_stride, out_row_stride, ignore_index, max_loss, vec));
+    FX_CHECK_LAUNCH("fx_softmax_ce");
+    return 0;
+}

@@ -1,0 +1,139 @@
+"""The LM head's fused forward + loss + backward over token micro-chunks, with the
+interface of flextrain/nn/head.py:60-393 (``LMHeadConfig``, ``LMHead.forward_backward``)
+and ``LossStats`` (flextrain/core/layer.py:1060-1088).
+
+Per micro-chunk: RMSNorm fwd -> logits GEMM -> loss fn (dZ in place) -> head
+weight-gradient GEMM (``beta = 1``, ``alpha = loss_scale``) -> dX GEMM -> RMSNorm
+bwd -> dx written over x.  The GEMMs go through the MFMA dispatcher; the
+weight may be stored ``(d_model, vocab)`` (reference) or be the transposed view
+of a ``(vocab, d_model)`` tensor (Hugging Face layout) without a copy.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Mapping, MutableMapping
+
+import torch
+
+from .loss import CrossEntropyLoss, LossFn, TokenContext
+from .matmul_dispatcher import CublasLtDispatcher
+from .ops.rmsnorm import flextrain_rmsnorm_bwd, flextrain_rmsnorm_fwd
+
+
+@dataclass(frozen=True)
+class LMHeadConfig:
+    """flextrain/nn/head.py:60-95 (the dtype-role fields feed the parameter
+    planner, which is outside this package, and are kept for signature parity)."""
+    d_model: int
+    vocab_size: int
+    rms_norm_eps: float = 1e-5
+    head_chunk_size: int = 1024
+    final_logit_softcap: float | None = None
+    compute_dtype: torch.dtype = torch.bfloat16
+    master_dtype: torch.dtype | None = None
+    grad_dtype: torch.dtype | None = None
+    norm_grad_dtype: torch.dtype = torch.float32
+    norm_master_dtype: torch.dtype = torch.float32
+    norm_compute_dtype: torch.dtype = torch.float32
+
+
+@dataclass
+class LossStats:
+    """flextrain/core/layer.py:1060-1088."""
+    per_token_loss: torch.Tensor
+    next_prediction: torch.Tensor
+    next_prediction_prob: torch.Tensor
+    token_count: int
+
+
+class LMHead:
+    layer_id: int = -2
+
+    def __init__(self, cfg: LMHeadConfig) -> None:
+        self.cfg = cfg
+        self._disp = None
+
+    def _dispatcher(self) -> CublasLtDispatcher:
+        if self._disp is None:
+            self._disp = CublasLtDispatcher(round_multiple=32)
+        return self._disp
+
+    def forward_backward(self, x, token_ctx: TokenContext, chunk, weights: Mapping[str, torch.Tensor],
+                         grads: MutableMapping[str, torch.Tensor], ctx, *, loss_scale: float = 1.0,
+                         loss_fn: LossFn | None = None):
+        """Returns ``(dx, stats)`` with ``dx is x`` (x is overwritten micro-chunk by
+        micro-chunk).  Gradients accumulate in place into ``grads["g_head_proj"]``
+        and ``grads["g_final_norm"]``; a missing/None entry skips that gradient.
+        flextrain/nn/head.py:155-393."""
+        if loss_fn is None:
+            loss_fn = CrossEntropyLoss()
+        num_tokens, d_model = x.shape
+        cfg = self.cfg
+        assert d_model == cfg.d_model, f"x has d_model={d_model}, head expects {cfg.d_model}"
+        if token_ctx.total_tokens != num_tokens:
+            raise ValueError(f"token_ctx covers {token_ctx.total_tokens} tokens, x has {num_tokens}")
+        device, dtype = x.device, x.dtype
+        per_token_loss = torch.empty(num_tokens, dtype=torch.float32, device=device)
+        next_prediction = torch.empty(num_tokens, dtype=torch.int64, device=device)
+        next_prediction_prob = torch.empty(num_tokens, dtype=torch.float32, device=device)
+        any_next_prediction = False
+        w_final_norm = weights["w_final_norm"]
+        w_head_proj = weights["w_head_proj"]                  # logical (d_model, vocab)
+        g_final_norm = grads.get("g_final_norm")
+        g_head_proj = grads.get("g_head_proj")
+        V = w_head_proj.shape[1]
+        disp = self._dispatcher()
+        stream = torch.cuda.current_stream(device).cuda_stream
+        aux_chunks = []
+        chunk_rows = min(cfg.head_chunk_size, num_tokens)
+        logits_buf = torch.empty((chunk_rows, V), dtype=dtype, device=device)
+        dx_head_buf = torch.empty((chunk_rows, d_model), dtype=dtype, device=device)
+
+        offset = 0
+        while offset < num_tokens:
+            t_prime = min(cfg.head_chunk_size, num_tokens - offset)
+            x_slice = x[offset:offset + t_prime]
+            head_in, rstd = flextrain_rmsnorm_fwd(x_slice, W=w_final_norm, rms_norm_eps=cfg.rms_norm_eps)
+            logits = logits_buf[:t_prime]
+            disp.matmul(stream, A=head_in, B=w_head_proj, D=logits)
+
+            cap = cfg.final_logit_softcap
+            softcap_gate = None
+            if cap is not None and cap > 0.0:
+                inv_cap = 1.0 / float(cap)
+                logits.mul_(inv_cap).tanh_().mul_(float(cap))
+                ratio = logits * inv_cap
+                softcap_gate = (1.0 - ratio * ratio).to(logits.dtype)
+
+            dZ, aux = loss_fn.compute(logits, token_ctx.slice_for(offset, t_prime), loss_scale=loss_scale,
+                                      per_token_loss_out=per_token_loss[offset:offset + t_prime])
+            if softcap_gate is not None:
+                dZ.mul_(softcap_gate)
+            if "next_prediction" in aux:
+                next_prediction[offset:offset + t_prime].copy_(aux.pop("next_prediction"))
+                next_prediction_prob[offset:offset + t_prime].copy_(aux.pop("next_prediction_prob"))
+                any_next_prediction = True
+            if aux:
+                aux_chunks.append(aux)
+
+            if g_head_proj is not None:
+                if g_head_proj.stride(1) == 1:      # (d, V) row-major: g += scale * h.T @ dZ
+                    disp.matmul(stream, A=head_in.T, B=dZ, C=g_head_proj, D=g_head_proj, alpha=loss_scale, beta=1.0)
+                else:                               # view of a (V, d) tensor: g.T += scale * dZ.T @ h
+                    g_t = g_head_proj.T
+                    disp.matmul(stream, A=dZ.T, B=head_in, C=g_t, D=g_t, alpha=loss_scale, beta=1.0)
+            dx_head = dx_head_buf[:t_prime]
+            disp.matmul(stream, A=dZ, B=w_head_proj.T, D=dx_head, alpha=loss_scale, beta=0.0)
+            dx_slice, _, _ = flextrain_rmsnorm_bwd(dx_head, x_slice, w_final_norm, rstd, dW=g_final_norm)
+            x_slice.copy_(dx_slice)
+            offset += t_prime
+
+        stats = LossStats(
+            per_token_loss=per_token_loss,
+            next_prediction=next_prediction if any_next_prediction else per_token_loss.new_empty(0, dtype=torch.int64),
+            next_prediction_prob=next_prediction_prob if any_next_prediction else per_token_loss.new_empty(0),
+            token_count=num_tokens,
+        )
+        if aux_chunks:
+            stats.aux_chunks = aux_chunks
+        return x, stats

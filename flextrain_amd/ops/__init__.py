@@ -27,6 +27,11 @@ from .rmsnorm import (
     flextrain_rmsnorm_fwd,
     flextrain_rmsnorm_fwd_recompute,
 )
+from .softmax_ce import (
+    flextrain_cross_entropy_loss,
+    flextrain_softmax,
+    flextrain_softmax_cross_entropy,
+)
 from .rope import (
     build_rope_inv_freq,
     flextrain_rope_bwd,
@@ -39,6 +44,7 @@ __all__ = [
     "build_rope_inv_freq",
     "flextrain_adamw_step",
     "flextrain_copy_expert_counts",
+    "flextrain_cross_entropy_loss",
     "flextrain_fused_topk_softmax",
     "flextrain_load_balance_bwd",
     "flextrain_moe_gather",
@@ -58,6 +64,8 @@ __all__ = [
     "flextrain_rope_fwd",
     "flextrain_rope_partial_bwd",
     "flextrain_rope_partial_fwd",
+    "flextrain_softmax",
+    "flextrain_softmax_cross_entropy",
     "flextrain_swiglu_bwd",
     "flextrain_swiglu_fwd",
 ]

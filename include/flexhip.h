@@ -184,6 +184,33 @@ int fx_swiglu_moe_bwd(void* dx, void* dw, int dw_dt, const void* dout, const voi
                       void* fwd_act, int64_t rows, int F, int64_t dx_row_stride, int64_t dout_row_stride,
                       int64_t x_row_stride, int64_t act_row_stride, int dt, int prescaled, hipStream_t stream);
 
+/* ---- Softmax / cross-entropy ------------------------------------------------ */
+
+/* flextrain_softmax (flextrain/ops/_kernels/softmax.py:111-215; kernel :13-108).
+ * out = softmax(x / temperature) per row, stored in out_dt.  max_idx_out
+ * (int64, first occurrence) and max_val_out (fp32, = 1/sum) are optional. */
+int fx_softmax(const void* x, void* out, int64_t* max_idx_out, float* max_val_out, int64_t rows, int V,
+               int64_t in_row_stride, int64_t out_row_stride, float temperature, int in_dt, int out_dt,
+               hipStream_t stream);
+
+/* flextrain_cross_entropy_loss (flextrain/ops/_kernels/cross_entropy.py:61-134;
+ * kernel :14-57).  probs is overwritten with dZ = P - onehot(label);
+ * loss_out[t] = min(-log P[t,label], max_loss), 0 for labels outside [0,V);
+ * valid_out[t] = 1/0. */
+int fx_cross_entropy(void* probs, const void* labels, int labels_are_int64, float* loss_out, float* valid_out,
+                     int64_t rows, int V, int64_t stride_t, int64_t stride_v, float max_loss, int dt,
+                     hipStream_t stream);
+
+/* CrossEntropyLoss.compute (flextrain/nn/loss.py:248-316) as one kernel: logits in,
+ * dZ out (dz_out may alias logits), per-row fp32 loss from the log-sum-exp
+ * (lse - logit[label], clamped to max_loss), rows with label == ignore_index or a
+ * zero loss_mask byte get loss 0 and a zero dZ row.  loss_mask (one byte per row),
+ * max_idx_out and max_val_out are optional. */
+int fx_softmax_ce(const void* logits, void* dz_out, const void* labels, int labels_are_int64,
+                  const uint8_t* loss_mask, float* loss_out, int64_t* max_idx_out, float* max_val_out, int64_t rows,
+                  int V, int64_t in_row_stride, int64_t out_row_stride, int64_t ignore_index, float max_loss, int dt,
+                  hipStream_t stream);
+
 /* ---- Expert-grouped GEMMs -------------------------------------------------- */
 
 /* Scratch bytes for the two grouped GEMM entry points (row offsets + tile list). */
