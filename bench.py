@@ -144,6 +144,139 @@ def run_extra(torch, ops, dev, stream, rn):
     rows.append(_op_entry("c4.adamw(fp32 p/m/v, bf16 g)", 26 * n, "GB/s", ms))
     del p, m, v, gr, pb
     torch.cuda.empty_cache()
+    rows += run_lm_head(torch, dev, stream, rn)
+    rows += run_moe(torch, dev, stream, rn)
+    return rows
+
+
+def run_lm_head(torch, dev, stream, rn):
+    """configs[2]: chunked linear cross-entropy fwd+bwd, hidden [8192,4096], lm_head
+    [128256,4096] (stored (V, d); the head sees the transposed view), chunk 1024."""
+    from flextrain_amd.head import LMHead, LMHeadConfig
+    from flextrain_amd.loss import TokenContext
+    from flextrain_amd.matmul_dispatcher import CublasLtDispatcher
+
+    T, d, V, chunk = 8192, 4096, 128256, 1024
+    x0 = rn(T, d).to(dev)
+    w = (torch.randn(V, d, device=dev) * 0.02).to(torch.bfloat16)
+    w_norm = torch.ones(d, dtype=torch.float32, device=dev)
+    labels = torch.randint(0, V, (T,), device=dev)
+    labels[torch.rand(T, device=dev) < 0.1] = -100
+    g_store = torch.zeros(V, d, dtype=torch.float32, device=dev)
+    g_norm = torch.zeros(d, dtype=torch.float32, device=dev)
+    head = LMHead(LMHeadConfig(d_model=d, vocab_size=V, head_chunk_size=chunk))
+    scale = 1.0 / int((labels != -100).sum())
+    x = x0.clone()
+
+    def run():
+        x.copy_(x0)
+        head.forward_backward(x, TokenContext(labels=labels), None, {"w_final_norm": w_norm, "w_head_proj": w.t()},
+                              {"g_head_proj": g_store.t(), "g_final_norm": g_norm}, None, loss_scale=scale)
+
+    rows = []
+    ms = _time_launches(torch, stream, [run], warmup=1, reps=3)
+    rows.append(_op_entry("c3.lm_head fwd+bwd (chunk 1024, fp32 dW)", 6 * T * d * V, "TFLOP/s", ms))
+    # the three GEMMs of one micro-chunk, timed alone
+    disp = CublasLtDispatcher()
+    sp = stream.cuda_stream
+    h = rn(chunk, d).to(dev)
+    logits = torch.empty(chunk, V, dtype=torch.bfloat16, device=dev)
+    dxh = torch.empty(chunk, d, dtype=torch.bfloat16, device=dev)
+    gt = g_store
+    ms = _time_launches(torch, stream, [lambda: disp.matmul_fast(sp, h, w.t(), D=logits)], warmup=2, reps=10)
+    rows.append(_op_entry("c3.logits gemm [1024,4096]x[4096,128256]", 2 * chunk * d * V, "TFLOP/s", ms))
+    logits.normal_()
+    ms = _time_launches(torch, stream, [lambda: disp.matmul_fast(sp, logits.t(), h, C=gt, D=gt, alpha=scale, beta=1.0)],
+                        warmup=2, reps=10)
+    rows.append(_op_entry("c3.dW gemm [128256,1024]x[1024,4096] (+= fp32)", 2 * chunk * d * V, "TFLOP/s", ms))
+    ms = _time_launches(torch, stream, [lambda: disp.matmul_fast(sp, logits, w, D=dxh)], warmup=2, reps=10)
+    rows.append(_op_entry("c3.dX gemm [1024,128256]x[128256,4096]", 2 * chunk * d * V, "TFLOP/s", ms))
+    from flextrain_amd import ops
+    lab = labels[:chunk].contiguous()
+    loss = torch.empty(chunk, dtype=torch.float32, device=dev)
+    ms = _time_launches(torch, stream, [lambda: ops.flextrain_softmax_cross_entropy(logits, lab, L=loss)], warmup=2, reps=10)
+    # two reads and one write of the logits chunk (the row does not stay in registers at V = 128256)
+    rows.append(_op_entry("c3.softmax_ce [1024,128256] in place", 3 * chunk * V * 2, "GB/s", ms))
+    del w, g_store, logits, x, x0
+    torch.cuda.empty_cache()
+    return rows
+
+
+def run_moe(torch, dev, stream, rn):
+    """configs[4]: Qwen3-30B-A3B-shaped routed-SwiGLU block fwd+bwd."""
+    import types
+
+    from flextrain_amd import full_moe
+    from flextrain_amd.moe_backend import FlextrainMoEExpertCompute
+    from flextrain_amd.ops.grouped import flextrain_grouped_gemm_rows, flextrain_grouped_gemm_wgrad
+
+    T, d, E, K, F = 8192, 2048, 128, 8, 768
+    TK = T * K
+    bf = torch.bfloat16
+    x, dy = rn(T, d).to(dev), rn(T, d).to(dev)
+    weights = dict(w_router=rn(d, E, std=0.02).to(dev),
+                   w_up=(torch.randn(E, 2 * F, d, device=dev) * 0.02).to(bf),
+                   w_down=(torch.randn(E, d, F, device=dev) * 0.02).to(bf))
+    grads = dict(g_router=torch.zeros(d, E, dtype=bf, device=dev), g_up=torch.zeros(E, 2 * F, d, dtype=bf, device=dev),
+                 g_down=torch.zeros(E, d, F, dtype=bf, device=dev))
+    slot = types.SimpleNamespace(
+        x_router=torch.empty(T, E, dtype=bf, device=dev), chosen_experts=torch.empty(T, K, dtype=torch.int32, device=dev),
+        router_weights=torch.empty(T, K, dtype=bf, device=dev), index_mapping=torch.empty(T, K, dtype=torch.int32, device=dev),
+        expert_counts=torch.empty(E, dtype=torch.int32, device=dev),
+        scattered_router_weights=torch.empty(TK, 1, dtype=bf, device=dev), x_up=torch.empty(TK, 2 * F, dtype=bf, device=dev),
+        aux={})
+    backend = FlextrainMoEExpertCompute()
+    pool = {}
+
+    def scratch(shape, dtype):   # a fixed scratch pool, as the engine's LayerContext provides
+        key = (tuple(shape), dtype, sum(1 for k in pool if k[:2] == (tuple(shape), dtype) and pool[k][1]))
+        if key not in pool:
+            pool[key] = [torch.empty(shape, dtype=dtype, device=dev), False]
+        pool[key][1] = True
+        return pool[key][0]
+
+    out = torch.empty(T, d, dtype=bf, device=dev)
+    extra = {}
+    common = dict(slot=slot, chunk_extra=extra, layer_id=0, primary_stream=stream, secondary_stream=None,
+                  scratch_fn=scratch, expert_compute=backend)
+
+    def release():
+        for v in pool.values():
+            v[1] = False
+
+    def fwd():
+        release()
+        full_moe.routed_swiglu_moe_fwd(x, weights, out_tensor=out, residual=x, top_k=K, num_experts=E,
+                                       routing_mode="topk_then_softmax", **common)
+
+    def bwd():
+        release()
+        full_moe.routed_swiglu_moe_bwd(dy, weights, grads, slot, extra, 0, ffn_norm_output=x, top_k=K, num_experts=E,
+                                       routing_mode="topk_then_softmax", load_balance_coef=0.0,
+                                       total_tokens_per_step=None, primary_stream=stream, secondary_stream=None,
+                                       scratch_fn=scratch, expert_compute=backend)
+
+    rows = []
+    fl_fwd = 6 * TK * d * F + 2 * T * d * E
+    fl_bwd = 12 * TK * d * F + 4 * T * d * E
+    ms_f = _time_launches(torch, stream, [fwd], warmup=2, reps=5)
+    rows.append(_op_entry("c5.moe block fwd (route+sort+scatter+experts+gather)", fl_fwd, "TFLOP/s", ms_f))
+    ms_b = _time_launches(torch, stream, [bwd], warmup=2, reps=5)
+    rows.append(_op_entry("c5.moe block bwd", fl_bwd, "TFLOP/s", ms_b))
+    rows.append(_op_entry("c5.moe block fwd+bwd", fl_fwd + fl_bwd, "TFLOP/s", ms_f + ms_b))
+    # the grouped GEMMs alone, on the routing the block just produced
+    counts = slot.expert_counts
+    sx = torch.randn(TK, d, device=dev).to(bf)
+    pre = slot.x_up
+    act = torch.randn(TK, F, device=dev).to(bf)
+    ms = _time_launches(torch, stream, [lambda: flextrain_grouped_gemm_rows(sx, weights["w_up"].transpose(1, 2), counts, pre)],
+                        warmup=2, reps=10)
+    rows.append(_op_entry("c5.grouped up-proj [65536,2048]x128x[2048,1536]", 2 * TK * d * 2 * F, "TFLOP/s", ms))
+    ms = _time_launches(torch, stream, [lambda: flextrain_grouped_gemm_rows(act, weights["w_down"].transpose(1, 2), counts, sx)],
+                        warmup=2, reps=10)
+    rows.append(_op_entry("c5.grouped down-proj [65536,768]x128x[768,2048]", 2 * TK * d * F, "TFLOP/s", ms))
+    ms = _time_launches(torch, stream, [lambda: flextrain_grouped_gemm_wgrad(pre, sx, grads["g_up"], counts)], warmup=2, reps=10)
+    rows.append(_op_entry("c5.grouped wgrad g_up [1536,T_e]x[T_e,2048] x128", 2 * TK * d * 2 * F, "TFLOP/s", ms))
     return rows
 
 
