@@ -7,7 +7,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import c_char_p, c_float, c_int, c_int32, c_int64, c_size_t, c_uint64, c_void_p, POINTER
+from ctypes import c_char_p, c_double, c_float, c_int, c_int32, c_int64, c_size_t, c_uint64, c_void_p, POINTER
 
 import torch
 
@@ -83,6 +83,9 @@ _SIGNATURES = {
     "dispatch_matmul": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int,
                                 c_void_p, c_int, c_void_p, c_int, c_void_p, c_size_t, c_int, c_int, c_int,
                                 c_int, c_int, c_float, c_float, c_int, c_int]),
+    "solve_scheduler": (c_double, [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_double, c_int, c_int,
+                                   c_void_p]),
+    "compute_buf_size": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p, c_double, c_int]),
     "fx_swiglu_moe_bwd": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                   c_int64, c_int, c_int64, c_int64, c_int64, c_int64, c_int, c_int,
                                   c_void_p]),

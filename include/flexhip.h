@@ -255,6 +255,24 @@ int dispatch_matmul(DispatchContext* ctx, intptr_t stream_ptr, int M, int N, int
                     intptr_t ptr_workspace, size_t workspace_bytes, int a_dt, int b_dt, int c_dt, int d_dt,
                     int compute_dt, float alpha, float beta, int trans_a, int trans_b);
 
+/* ---- Save-level transmission scheduler (verbatim ABI of the reference helper) -- */
+
+/* helpers/transmission_scheduler/transmission_scheduler/transmission_scheduler.h:23-36
+ * (implementation transmission_scheduler.c:25-457).  Host code, no GPU work.
+ * T tasks, N buffers, k options per task; compute (T), durations and sizes (T*k,
+ * row-major) in milliseconds / arbitrary value units; time_scale ticks per
+ * millisecond; buf_size from compute_buf_size.  Writes the chosen option of every
+ * task to out_choices (T ints) and returns the maximal total value, or 0.0 when
+ * no schedule meets the deadlines (out_choices is then left untouched). */
+double solve_scheduler(int T, int N, int k, const double* compute, const double* durations,
+                       const double* sizes, double deadline, int time_scale, int buf_size,
+                       int* out_choices);
+
+/* transmission_scheduler.h:38-40 (transmission_scheduler.c:463-533): window width
+ * for solve_scheduler, a power of two >= 2048. */
+int compute_buf_size(int T, int N, int k, const double* compute, const double* durations, double deadline,
+                     int time_scale);
+
 #ifdef __cplusplus
 }
 #endif

@@ -21,4 +21,11 @@ How each function is pinned (tests/test_oracle_*.py, all CPU-only):
                torch.autograd of those (tests/test_gelu_tanh_gated_kernel.py:57-89).
   adamw        torch.optim.AdamW run for several steps
                (flextrain/bench/parity.py:546-577) and the step-1 closed form.
+  linear_ce    torch.softmax / argmax, F.cross_entropy (none / sum, ignore_index),
+               torch.autograd through rms_norm -> matmul -> cross-entropy.
+  moe          stable sort / bincount / indexing identities, torch.autograd through
+               the eager expert formula (tests/moe/test_moe_backend_parity.py:45-107).
+  dp_solver    golden vectors from the compiled reference solver (oracle/_ref, built
+               by oracle/Makefile from the reference's own C file), the README known
+               answer, exhaustive enumeration of all option vectors on small problems.
 """
