@@ -83,6 +83,15 @@ _SIGNATURES = {
     "dispatch_matmul": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int,
                                 c_void_p, c_int, c_void_p, c_int, c_void_p, c_size_t, c_int, c_int, c_int,
                                 c_int, c_int, c_float, c_float, c_int, c_int]),
+    "fx_host_alloc": (c_int, [c_size_t, POINTER(c_void_p)]),
+    "fx_host_free": (c_int, [c_void_p]),
+    "fx_host_register": (c_int, [c_void_p, c_size_t]),
+    "fx_host_unregister": (c_int, [c_void_p]),
+    "fx_adamw_stream_ws_bytes": (c_size_t, [c_int64, c_int, c_int, c_int, c_int, c_int]),
+    "fx_adamw_stream_chunk": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int,
+                                      c_int, c_int, c_float, c_float, c_float, c_float, c_float, c_float,
+                                      c_float, c_void_p, c_size_t, c_int64, c_int, c_void_p, c_void_p,
+                                      c_void_p]),
     "solve_scheduler": (c_double, [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_double, c_int, c_int,
                                    c_void_p]),
     "compute_buf_size": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p, c_double, c_int]),

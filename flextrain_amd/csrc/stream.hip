@@ -1,0 +1,186 @@
+// Host <-> HBM streaming of one offloaded optimizer chunk, and pinned host memory.
+//
+// The reference engine keeps master weights, gradients and Adam moments of a layer in
+// pinned host memory and, for the optimizer step, copies a whole layer in on an
+// "inbound" stream, runs one kernel per tensor on the "compute" stream and copies the
+// layer back on an "outbound" stream, rotating layers through ring slots
+// (flextrain/engine/active_model.py:486-655, flextrain/engine/buffers.py:1088-1291,
+// streams of flextrain/engine/streams.py:85-128).  fx_adamw_stream_chunk does the same
+// for ONE flat chunk at a finer grain: the chunk is cut into sub-chunks that rotate
+// through n_slots device staging slots, so the copy-in of sub-chunk i+1, the kernel of
+// sub-chunk i and the copy-out of sub-chunk i-1 overlap and both PCIe directions stay
+// busy.  Everything is enqueued without blocking the host; ordering is by events:
+//     copy-in(i)  waits for copy-out(i - n_slots)     (the slot is free again)
+//     kernel(i)   waits for copy-in(i)
+//     copy-out(i) waits for kernel(i)
+// Pinned host memory comes from hipHostMalloc (exact size, no power-of-two rounding:
+// the reason the reference registers plain allocations instead of using the caching
+// pinned allocator, flextrain/engine/host_memory.py:161-176).
+#include "common.h"
+#include "flexhip.h"
+
+using namespace fx;
+
+namespace {
+
+inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+struct SlotLayout {
+    size_t p, g, m, v, pc, stride;  // byte offsets inside a slot, slot stride
+};
+
+SlotLayout slot_layout(int64_t sub, int p_dt, int g_dt, int s_dt, bool staged_copy) {
+    SlotLayout L;
+    size_t o = 0;
+    L.p = o;  o = align_up(o + (size_t)sub * elem_size(p_dt), 256);
+    L.g = o;  o = align_up(o + (size_t)sub * elem_size(g_dt), 256);
+    L.m = o;  o = align_up(o + (size_t)sub * elem_size(s_dt), 256);
+    L.v = o;  o = align_up(o + (size_t)sub * elem_size(s_dt), 256);
+    L.pc = o; if (staged_copy) o = align_up(o + (size_t)sub * 2, 256);
+    L.stride = o;
+    return L;
+}
+
+#define FX_HIP_OK(expr, what)                                                          \
+    do {                                                                               \
+        hipError_t e__ = (expr);                                                       \
+        if (e__ != hipSuccess) {                                                       \
+            fprintf(stderr, "flexhip: %s: %s\n", what, hipGetErrorString(e__));        \
+            rc = -1;                                                                   \
+            goto done;                                                                 \
+        }                                                                              \
+    } while (0)
+
+}  // namespace
+
+extern "C" size_t fx_adamw_stream_ws_bytes(int64_t sub_elems, int n_slots, int p_dt, int g_dt, int state_dt,
+                                           int stage_bf16_copy) {
+    if (sub_elems <= 0 || n_slots <= 0) return 0;
+    return slot_layout(sub_elems, p_dt, g_dt, state_dt, stage_bf16_copy != 0).stride * (size_t)n_slots;
+}
+
+extern "C" int fx_adamw_stream_chunk(void* p_host, const void* g_host, void* m_host, void* v_host,
+                                     void* p_bf16_out, int p_bf16_out_on_device, int64_t n, int p_dt, int g_dt,
+                                     int state_dt, float lr, float beta1, float beta2, float eps, float weight_decay,
+                                     float bias_correction1, float bias_correction2, void* ws, size_t ws_bytes,
+                                     int64_t sub_elems, int n_slots, hipStream_t inbound, hipStream_t compute,
+                                     hipStream_t outbound) {
+    if (n < 0) FX_FAIL("fx_adamw_stream_chunk: negative element count");
+    if (n == 0) return 0;
+    if (!p_host || !g_host || !m_host || !v_host || !ws) FX_FAIL("fx_adamw_stream_chunk: null pointer");
+    if (sub_elems <= 0 || (sub_elems & 7) || n_slots < 1 || n_slots > 16)
+        FX_FAIL("fx_adamw_stream_chunk: sub_elems must be a positive multiple of 8 and 1 <= n_slots <= 16");
+    if (!inbound || !compute || !outbound) FX_FAIL("fx_adamw_stream_chunk: the three streams must be explicit (non-null)");
+    if (!aligned16(ws) || !aligned16(p_host) || !aligned16(g_host) || !aligned16(m_host) || !aligned16(v_host) ||
+        (p_bf16_out && !aligned16(p_bf16_out)))
+        FX_FAIL("fx_adamw_stream_chunk: buffers must be 16-byte aligned");
+    const bool stage_copy = p_bf16_out && !p_bf16_out_on_device;
+    const SlotLayout L = slot_layout(sub_elems, p_dt, g_dt, state_dt, stage_copy);
+    if (ws_bytes < L.stride * (size_t)n_slots)
+        FX_FAIL("fx_adamw_stream_chunk: workspace too small (%zu < %zu bytes)", ws_bytes, L.stride * (size_t)n_slots);
+
+    const size_t psz = elem_size(p_dt), gsz = elem_size(g_dt), ssz = elem_size(state_dt);
+    hipEvent_t in_done[16], k_done[16], out_done[16];
+    int made = 0, rc = 0;
+    for (; made < n_slots; ++made) {
+        if (hipEventCreateWithFlags(&in_done[made], hipEventDisableTiming) != hipSuccess ||
+            hipEventCreateWithFlags(&k_done[made], hipEventDisableTiming) != hipSuccess ||
+            hipEventCreateWithFlags(&out_done[made], hipEventDisableTiming) != hipSuccess) {
+            fprintf(stderr, "flexhip: fx_adamw_stream_chunk: event creation failed\n");
+            return -1;  // events of earlier slots leak only on this failure path
+        }
+    }
+    {
+        char* base = reinterpret_cast<char*>(ws);
+        char* ph = reinterpret_cast<char*>(p_host);
+        const char* gh = reinterpret_cast<const char*>(g_host);
+        char* mh = reinterpret_cast<char*>(m_host);
+        char* vh = reinterpret_cast<char*>(v_host);
+        char* ch = reinterpret_cast<char*>(p_bf16_out);
+        int64_t i = 0;
+        for (int64_t off = 0; off < n; off += sub_elems, ++i) {
+            const int64_t cnt = (n - off < sub_elems) ? (n - off) : sub_elems;
+            const int s = (int)(i % n_slots);
+            char* slot = base + (size_t)s * L.stride;
+            if (i >= n_slots) FX_HIP_OK(hipStreamWaitEvent(inbound, out_done[s], 0), "wait for a free slot");
+            FX_HIP_OK(hipMemcpyAsync(slot + L.p, ph + off * psz, cnt * psz, hipMemcpyHostToDevice, inbound), "copy-in p");
+            FX_HIP_OK(hipMemcpyAsync(slot + L.g, gh + off * gsz, cnt * gsz, hipMemcpyHostToDevice, inbound), "copy-in g");
+            FX_HIP_OK(hipMemcpyAsync(slot + L.m, mh + off * ssz, cnt * ssz, hipMemcpyHostToDevice, inbound), "copy-in m");
+            FX_HIP_OK(hipMemcpyAsync(slot + L.v, vh + off * ssz, cnt * ssz, hipMemcpyHostToDevice, inbound), "copy-in v");
+            FX_HIP_OK(hipEventRecord(in_done[s], inbound), "record copy-in");
+
+            FX_HIP_OK(hipStreamWaitEvent(compute, in_done[s], 0), "wait for copy-in");
+            void* copy_dst = nullptr;
+            if (p_bf16_out) copy_dst = stage_copy ? (void*)(slot + L.pc) : (void*)(ch + off * 2);
+            if (fx_adamw_step(slot + L.p, slot + L.g, slot + L.m, slot + L.v, copy_dst, cnt, p_dt, g_dt, state_dt, lr,
+                              beta1, beta2, eps, weight_decay, bias_correction1, bias_correction2, compute) != 0) {
+                rc = -1;
+                goto done;
+            }
+            FX_HIP_OK(hipEventRecord(k_done[s], compute), "record kernel");
+
+            FX_HIP_OK(hipStreamWaitEvent(outbound, k_done[s], 0), "wait for the kernel");
+            FX_HIP_OK(hipMemcpyAsync(ph + off * psz, slot + L.p, cnt * psz, hipMemcpyDeviceToHost, outbound), "copy-out p");
+            FX_HIP_OK(hipMemcpyAsync(mh + off * ssz, slot + L.m, cnt * ssz, hipMemcpyDeviceToHost, outbound), "copy-out m");
+            FX_HIP_OK(hipMemcpyAsync(vh + off * ssz, slot + L.v, cnt * ssz, hipMemcpyDeviceToHost, outbound), "copy-out v");
+            if (stage_copy)
+                FX_HIP_OK(hipMemcpyAsync(ch + off * 2, slot + L.pc, cnt * 2, hipMemcpyDeviceToHost, outbound), "copy-out bf16 p");
+            FX_HIP_OK(hipEventRecord(out_done[s], outbound), "record copy-out");
+        }
+    }
+done:
+    // Destroying an event that is still pending is allowed: its resources are released
+    // when it completes.
+    for (int s = 0; s < made; ++s) {
+        (void)hipEventDestroy(in_done[s]);
+        (void)hipEventDestroy(k_done[s]);
+        (void)hipEventDestroy(out_done[s]);
+    }
+    return rc;
+}
+
+extern "C" int fx_host_alloc(size_t bytes, void** out) {
+    if (!out) FX_FAIL("fx_host_alloc: null output pointer");
+    *out = nullptr;
+    if (bytes == 0) return 0;
+    hipError_t e = hipHostMalloc(out, bytes, hipHostMallocDefault);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        FX_FAIL("fx_host_alloc: hipHostMalloc(%zu) failed: %s", bytes, hipGetErrorString(e));
+    }
+    return 0;
+}
+
+extern "C" int fx_host_free(void* ptr) {
+    if (!ptr) return 0;
+    hipError_t e = hipHostFree(ptr);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        FX_FAIL("fx_host_free: %s", hipGetErrorString(e));
+    }
+    return 0;
+}
+
+extern "C" int fx_host_register(void* ptr, size_t bytes) {
+    if (!ptr || bytes == 0) return 0;
+    hipError_t e = hipHostRegister(ptr, bytes, hipHostRegisterDefault);
+    if (e == hipErrorHostMemoryAlreadyRegistered) {
+        (void)hipGetLastError();  // benign, and must not surface on the next HIP call
+        return 1;
+    }
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        FX_FAIL("fx_host_register: hipHostRegister(%zu bytes) failed: %s", bytes, hipGetErrorString(e));
+    }
+    return 0;
+}
+
+extern "C" int fx_host_unregister(void* ptr) {
+    if (!ptr) return 0;
+    hipError_t e = hipHostUnregister(ptr);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        FX_FAIL("fx_host_unregister: %s", hipGetErrorString(e));
+    }
+    return 0;
+}

@@ -255,6 +255,46 @@ int dispatch_matmul(DispatchContext* ctx, intptr_t stream_ptr, int M, int N, int
                     intptr_t ptr_workspace, size_t workspace_bytes, int a_dt, int b_dt, int c_dt, int d_dt,
                     int compute_dt, float alpha, float beta, int trans_a, int trans_b);
 
+/* ---- Pinned host memory and the streamed optimizer chunk -------------------- */
+
+/* Pinned (page-locked, device-visible) host memory of exactly `bytes` bytes.  Stands in
+ * for the allocate-then-cudaHostRegister sequence of
+ * flextrain/engine/host_memory.py:76-100, :178-212 and
+ * flextrain/ops/_kernels/_mem_register.py:4-9 on systems where registering memory that
+ * already exists is not permitted.  *out receives the pointer (NULL for 0 bytes). */
+int fx_host_alloc(size_t bytes, void** out);
+int fx_host_free(void* ptr);
+
+/* cudaHostRegister / cudaHostUnregister of flextrain/ops/_kernels/_mem_register.py:4-20
+ * and flextrain/engine/host_memory.py:76-106.  fx_host_register returns 0 on a fresh
+ * registration, 1 when the range was already registered (benign, as the reference
+ * treats error 712), -1 on failure; a failure leaves no pending HIP error behind. */
+int fx_host_register(void* ptr, size_t bytes);
+int fx_host_unregister(void* ptr);
+
+/* Device staging bytes fx_adamw_stream_chunk needs for n_slots slots of sub_elems
+ * elements (p, g, m, v and, when stage_bf16_copy, the bf16 copy of p). */
+size_t fx_adamw_stream_ws_bytes(int64_t sub_elems, int n_slots, int p_dt, int g_dt, int state_dt,
+                                int stage_bf16_copy);
+
+/* The optimizer step of one host-offloaded chunk: the fetch / step / offload pipeline of
+ * ActiveModel.step (flextrain/engine/active_model.py:486-655) with
+ * BufferManager.fetch_layer_{params,grads,opt} / offload_layer_{params,opt}
+ * (flextrain/engine/buffers.py:1088-1291) for one flat chunk of n elements.
+ * p_host, g_host, m_host, v_host: pinned host memory (p, m, v are updated in place).
+ * p_bf16_out: optional bf16 copy of the updated parameters, in pinned host memory
+ * (p_bf16_out_on_device = 0) or in device memory (1).  The chunk moves through n_slots
+ * (1..16) device slots of sub_elems (multiple of 8) elements inside ws; copies in run on
+ * `inbound`, kernels on `compute`, copies out on `outbound` (three distinct non-null
+ * streams give full overlap).  Enqueues only: the host buffers hold the result once
+ * `outbound` (and, for a device-side bf16 copy, `compute`) has drained.  The caller
+ * orders the three streams after whatever produced the host buffers. */
+int fx_adamw_stream_chunk(void* p_host, const void* g_host, void* m_host, void* v_host, void* p_bf16_out,
+                          int p_bf16_out_on_device, int64_t n, int p_dt, int g_dt, int state_dt, float lr,
+                          float beta1, float beta2, float eps, float weight_decay, float bias_correction1,
+                          float bias_correction2, void* ws, size_t ws_bytes, int64_t sub_elems, int n_slots,
+                          hipStream_t inbound, hipStream_t compute, hipStream_t outbound);
+
 /* ---- Save-level transmission scheduler (verbatim ABI of the reference helper) -- */
 
 /* helpers/transmission_scheduler/transmission_scheduler/transmission_scheduler.h:23-36
