@@ -6,13 +6,13 @@
 // (create_dispatcher / destroy_dispatcher / get_stats / dispatch_matmul).  The
 // reference asks cuBLASLt for an algorithm and caches it per exact shape and per
 // rounded ("fuzzy") shape; here the cached "algorithm" is the tile shape of the
-// hand-written MFMA kernel in gemm_core.h, chosen by a fill heuristic, and the
+// hand-written MFMA kernel in gemm_core2.h, chosen by a fill heuristic, and the
 // cache/statistics bookkeeping keeps the same meaning (exact hit, fuzzy hit,
 // new algorithm saved).
 #include <chrono>
 #include <unordered_map>
 
-#include "gemm_core.h"
+#include "gemm_core2.h"
 #include "flexhip.h"
 
 namespace fx {
@@ -39,17 +39,43 @@ FX_DEV void tile_coords(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
     tn = (p % width) / gsz;
 }
 
-template <typename T, typename TD, int BM, int BN, bool A_MN, bool B_MN>
-__global__ __launch_bounds__(GEMM_THREADS) void gemm_kernel(
-    const T* __restrict__ A, const T* __restrict__ B, const TD* C, TD* D, int M, int N, int K, int64_t lda,
-    int64_t ldb, int64_t ldc, int64_t ldd, float alpha, float beta, int tiles_m, int tiles_n) {
+// blockIdx.y selects a K split: split s covers k in [s*k_per_split, min(K, (s+1)*k_per_split)) and,
+// when there is more than one, writes its fp32 partial product to PART + s*M*N (row stride N).
+template <typename T, typename TD, int BM, int BN, int WAVES_M, int WAVES_N, bool A_MN, bool B_MN>
+__global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_kernel(
+    const T* __restrict__ A, const T* __restrict__ B, const TD* C, TD* D, float* PART, int M, int N, int K,
+    int k_per_split, int64_t lda, int64_t ldb, int64_t ldc, int64_t ldd, float alpha, float beta, int tiles_m,
+    int tiles_n) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T* smem = reinterpret_cast<T*>(smem_raw);
     int tm, tn;
     tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
-    OperandView<T> a{A, lda, M, tm * BM};
-    OperandView<T> b{B, ldb, N, tn * BN};
-    gemm_tile<T, TD, BM, BN, A_MN, B_MN>(a, b, C, D, ldc, ldd, M, N, K, 0, alpha, beta, smem);
+    const int k0 = blockIdx.y * k_per_split;
+    const int klen = (K - k0) < k_per_split ? (K - k0) : k_per_split;
+    OperandView<T> a{A + (A_MN ? (int64_t)k0 * lda : (int64_t)k0), lda, M, tm * BM};
+    OperandView<T> b{B + (B_MN ? (int64_t)k0 * ldb : (int64_t)k0), ldb, N, tn * BN};
+    if (gridDim.y == 1) {
+        gemm_tile2<T, TD, BM, BN, WAVES_M, WAVES_N, A_MN, B_MN>(a, b, C, D, ldc, ldd, M, N, klen, alpha, beta, smem);
+    } else {
+        float* part = PART + (int64_t)blockIdx.y * M * N;
+        gemm_tile2<T, float, BM, BN, WAVES_M, WAVES_N, A_MN, B_MN>(a, b, nullptr, part, N, N, M, N, klen, 1.f, 0.f, smem);
+    }
+}
+
+// D = alpha * sum_s PART[s] + beta * C over M x N, 8 elements per lane (N % 8 == 0 is not required).
+template <typename TD>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ PART, int splits, const TD* C,
+                                                           TD* D, int M, int N, int64_t ldc, int64_t ldd,
+                                                           float alpha, float beta) {
+    const int64_t total = (int64_t)M * N;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        float acc = 0.f;
+        for (int s = 0; s < splits; ++s) acc += PART[(int64_t)s * total + i];
+        const int m = (int)(i / N), n = (int)(i % N);
+        float r = alpha * acc;
+        if (beta != 0.f) r += beta * (float)C[(int64_t)m * ldc + n];
+        D[(int64_t)m * ldd + n] = (TD)r;
+    }
 }
 
 // Any dtype / alignment: one output element per lane.  Correct, not fast.
@@ -75,27 +101,60 @@ enum TileCfg : int { TILE_256x256 = 0, TILE_256x128 = 1, TILE_128x128 = 2, TILE_
 
 static inline int cdiv(int a, int b) { return (a + b - 1) / b; }
 
-// Largest tile that still gives every CU at least one workgroup.
+// Largest tile that still gives (nearly) every CU a workgroup.
 static TileCfg choose_tile(int M, int N) {
     const long cus = 256;
-    if ((long)cdiv(M, 256) * cdiv(N, 256) >= cus) return TILE_256x256;
+    if ((long)cdiv(M, 256) * cdiv(N, 256) >= cus * 3 / 4) return TILE_256x256;
     if ((long)cdiv(M, 256) * cdiv(N, 128) >= cus) return TILE_256x128;
     return TILE_128x128;
 }
 
-template <typename T, typename TD, int BM, int BN>
-static void launch_tile(const void* A, const void* B, const void* C, void* D, int M, int N, int K, int64_t lda,
-                        int64_t ldb, int64_t ldc, int64_t ldd, float alpha, float beta, int ta, int tb,
-                        hipStream_t s) {
+// K splits for problems whose output has too few tiles to fill the GPU (e.g. the LM-head dX GEMM,
+// 1024 x 4096 with K = 128256): the largest tile, K cut into `splits` ranges of a multiple of 64.
+static int choose_splits(int M, int N, int K, size_t workspace_bytes) {
+    const long tiles = (long)cdiv(M, 256) * cdiv(N, 256);
+    if (tiles >= 128 || K < 4096) return 1;
+    long s = 256 / tiles;
+    if (s > K / 2048) s = K / 2048;
+    const size_t per = (size_t)M * N * sizeof(float);
+    if (per == 0 || (size_t)s * per > workspace_bytes) s = (long)(workspace_bytes / (per ? per : 1));
+    if (s > 16) s = 16;
+    return s < 2 ? 1 : (int)s;
+}
+
+template <typename T, typename TD, int BM, int BN, int WAVES_M, int WAVES_N, bool A_MN, bool B_MN>
+static void launch_one(const T* a, const T* b, const TD* c, TD* d, float* part, int splits, int M, int N, int K,
+                       int64_t lda, int64_t ldb, int64_t ldc, int64_t ldd, float alpha, float beta, hipStream_t s) {
+    auto kern = gemm_kernel<T, TD, BM, BN, WAVES_M, WAVES_N, A_MN, B_MN>;
+    constexpr size_t lds = gemm2_lds_bytes<T, BM, BN, WAVES_M, WAVES_N>();
+    static bool attr_set = false;  // more than 64 KB of dynamic LDS has to be asked for once per kernel
+    if (!attr_set) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        attr_set = true;
+    }
     const int tiles_m = cdiv(M, BM), tiles_n = cdiv(N, BN);
-    const unsigned grid = (unsigned)(tiles_m * tiles_n);
-    const size_t lds = (size_t)(BM + BN) * GEMM_BK * sizeof(T);
+    int k_per_split = K;
+    if (splits > 1) k_per_split = cdiv(cdiv(K, splits), GEMM_BK) * GEMM_BK;
+    const int nsplit = cdiv(K, k_per_split);
+    kern<<<dim3((unsigned)(tiles_m * tiles_n), (unsigned)nsplit), WAVES_M * WAVES_N * 64, lds, s>>>(
+        a, b, c, d, part, M, N, K, k_per_split, lda, ldb, ldc, ldd, alpha, beta, tiles_m, tiles_n);
+    if (nsplit > 1) {
+        const int64_t total = (int64_t)M * N;
+        const unsigned grid = (unsigned)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
+        splitk_reduce_kernel<TD><<<grid, 256, 0, s>>>(part, nsplit, c, d, M, N, ldc, ldd, alpha, beta);
+    }
+}
+
+template <typename T, typename TD, int BM, int BN, int WAVES_M, int WAVES_N>
+static void launch_tile(const void* A, const void* B, const void* C, void* D, float* part, int splits, int M, int N,
+                        int K, int64_t lda, int64_t ldb, int64_t ldc, int64_t ldd, float alpha, float beta, int ta,
+                        int tb, hipStream_t s) {
     const T* a = reinterpret_cast<const T*>(A);
     const T* b = reinterpret_cast<const T*>(B);
     const TD* c = reinterpret_cast<const TD*>(C);
     TD* d = reinterpret_cast<TD*>(D);
     // operand form: A is MN-contiguous when transposed, B when NOT transposed
-#define FX_GEMM_GO(AM, BMN) gemm_kernel<T, TD, BM, BN, AM, BMN><<<grid, GEMM_THREADS, lds, s>>>(a, b, c, d, M, N, K, lda, ldb, ldc, ldd, alpha, beta, tiles_m, tiles_n)
+#define FX_GEMM_GO(AM, BMN) launch_one<T, TD, BM, BN, WAVES_M, WAVES_N, AM, BMN>(a, b, c, d, part, splits, M, N, K, lda, ldb, ldc, ldd, alpha, beta, s)
     if (!ta && tb) FX_GEMM_GO(false, false);
     else if (!ta && !tb) FX_GEMM_GO(false, true);
     else if (ta && tb) FX_GEMM_GO(true, false);
@@ -104,12 +163,14 @@ static void launch_tile(const void* A, const void* B, const void* C, void* D, in
 }
 
 template <typename T, typename TD>
-static void launch_cfg(TileCfg cfg, const void* A, const void* B, const void* C, void* D, int M, int N, int K,
+static void launch_cfg(int cfg, const void* A, const void* B, const void* C, void* D, float* part, int M, int N, int K,
                        int64_t lda, int64_t ldb, int64_t ldc, int64_t ldd, float alpha, float beta, int ta,
                        int tb, hipStream_t s) {
-    if (cfg == TILE_256x256) launch_tile<T, TD, 256, 256>(A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, ta, tb, s);
-    else if (cfg == TILE_256x128) launch_tile<T, TD, 256, 128>(A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, ta, tb, s);
-    else launch_tile<T, TD, 128, 128>(A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, ta, tb, s);
+    const int tile = cfg & 0xff, splits = cfg >> 8;
+    // 8 waves (two per SIMD) on the largest tile, 4 on the smaller ones
+    if (tile == TILE_256x256) launch_tile<T, TD, 256, 256, 4, 2>(A, B, C, D, part, splits, M, N, K, lda, ldb, ldc, ldd, alpha, beta, ta, tb, s);
+    else if (tile == TILE_256x128) launch_tile<T, TD, 256, 128, 2, 2>(A, B, C, D, part, splits, M, N, K, lda, ldb, ldc, ldd, alpha, beta, ta, tb, s);
+    else launch_tile<T, TD, 128, 128, 2, 2>(A, B, C, D, part, splits, M, N, K, lda, ldb, ldc, ldd, alpha, beta, ta, tb, s);
 }
 
 // Can the MFMA path take this problem?  16-byte aligned operands whose
@@ -188,7 +249,8 @@ extern "C" int dispatch_matmul(DispatchContext* ctx, intptr_t stream_ptr, int M,
                                int ldd, intptr_t ptr_workspace, size_t workspace_bytes, int a_dt, int b_dt,
                                int c_dt, int d_dt, int compute_dt, float alpha, float beta, int trans_a,
                                int trans_b) {
-    (void)ptr_workspace; (void)workspace_bytes; (void)compute_dt;  // fp32 compute always; no workspace needed
+    (void)compute_dt;  // fp32 accumulation always
+    float* part = reinterpret_cast<float*>(ptr_workspace);  // split-K partial sums, when the caller lends a workspace
     const uint64_t t0 = now_ns();
     if (M == 0 || N == 0 || K == 0) return 0;  // no-op, as the reference (dispatch.cpp:161)
     if (!ctx) FX_FAIL("dispatch_matmul: null dispatcher");
@@ -226,8 +288,14 @@ extern "C" int dispatch_matmul(DispatchContext* ctx, intptr_t stream_ptr, int M,
             ctx->fuzzy[fk] = cfg;
             ctx->algos_saved++;
         }
+        if (cfg != TILE_GENERIC && part && (reinterpret_cast<uintptr_t>(part) & 15u) == 0) {
+            const int splits = choose_splits(M, N, K, workspace_bytes);   // depends on the exact shape: kept out of the fuzzy cache
+            if (splits > 1) cfg = TILE_256x256 | (splits << 8);
+        }
         ctx->exact[key] = cfg;
     }
+    if ((cfg >> 8) > 1 && (!part || (size_t)(cfg >> 8) * M * N * sizeof(float) > workspace_bytes))
+        cfg &= 0xff;  // cached with K splits, but this call lends no (or too small a) workspace
     const uint64_t h2 = now_ns();
 
     if (cfg == TILE_GENERIC) {
@@ -241,11 +309,11 @@ extern "C" int dispatch_matmul(DispatchContext* ctx, intptr_t stream_ptr, int M,
                     reinterpret_cast<const TA*>(A), reinterpret_cast<const TA*>(B), reinterpret_cast<const TD*>(C),
                     reinterpret_cast<TD*>(D), M, N, K, lda, ldb, ldc, ldd, alpha, beta, trans_a, trans_b)));
     } else if (a_dt == DT_BF16 && d_dt == DT_BF16) {
-        launch_cfg<bf16, bf16>((TileCfg)cfg, A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, trans_a, trans_b, stream);
+        launch_cfg<bf16, bf16>(cfg, A, B, C, D, part, M, N, K, lda, ldb, ldc, ldd, alpha, beta, trans_a, trans_b, stream);
     } else if (a_dt == DT_BF16) {
-        launch_cfg<bf16, float>((TileCfg)cfg, A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, trans_a, trans_b, stream);
+        launch_cfg<bf16, float>(cfg, A, B, C, D, part, M, N, K, lda, ldb, ldc, ldd, alpha, beta, trans_a, trans_b, stream);
     } else {
-        launch_cfg<f16, f16>((TileCfg)cfg, A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, trans_a, trans_b, stream);
+        launch_cfg<f16, f16>(cfg, A, B, C, D, part, M, N, K, lda, ldb, ldc, ldd, alpha, beta, trans_a, trans_b, stream);
     }
     const uint64_t h3 = now_ns();
     ctx->hash_ns += h1 - h0;

@@ -11,7 +11,7 @@
 //
 // where rows of expert e are the contiguous range [off_e, off_e + c_e) of the
 // expert-sorted buffers and off = exclusive prefix sum of the counts.
-#include "gemm_core.h"
+#include "gemm_core2.h"
 #include "flexhip.h"
 
 namespace fx {
@@ -68,8 +68,8 @@ __global__ __launch_bounds__(256) void grouped_plan_kernel(const int32_t* __rest
     if (threadIdx.x == 0) { OFFSETS[E] = carry_r; NTILES[0] = carry_t; }
 }
 
-template <typename T, int BM, int BN, bool B_MN>
-__global__ __launch_bounds__(GEMM_THREADS) void grouped_rows_kernel(
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool B_MN>
+__global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void grouped_rows_kernel(
     const T* __restrict__ A, int64_t lda, const T* __restrict__ B, int64_t ldb, int64_t b_expert_stride,
     const T* C, int64_t ldc, T* D, int64_t ldd, const int32_t* __restrict__ NTILES,
     const int32_t* __restrict__ OFFSETS, const int32_t* __restrict__ TILES, int N, int K, float alpha,
@@ -85,11 +85,11 @@ __global__ __launch_bounds__(GEMM_THREADS) void grouped_rows_kernel(
     OperandView<T> a{A + row0 * lda, lda, rows, m0};
     OperandView<T> b{B + (int64_t)e * b_expert_stride, ldb, N, (int)blockIdx.y * BN};
     const T* c = C ? C + row0 * ldc : nullptr;
-    gemm_tile<T, T, BM, BN, false, B_MN>(a, b, c, D + row0 * ldd, ldc, ldd, rows, N, K, 0, alpha, beta, smem);
+    gemm_tile2<T, T, BM, BN, WAVES_M, WAVES_N, false, B_MN>(a, b, c, D + row0 * ldd, ldc, ldd, rows, N, K, alpha, beta, smem);
 }
 
-template <typename T, typename TG, int BM, int BN>
-__global__ __launch_bounds__(GEMM_THREADS) void grouped_wgrad_kernel(
+template <typename T, typename TG, int BM, int BN, int WAVES_M, int WAVES_N>
+__global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void grouped_wgrad_kernel(
     const T* __restrict__ A, int64_t lda, const T* __restrict__ B, int64_t ldb, TG* G, int64_t ldg,
     int64_t g_expert_stride, const int32_t* __restrict__ OFFSETS, int M, int N, float alpha, float beta,
     int tiles_n) {
@@ -103,7 +103,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void grouped_wgrad_kernel(
     OperandView<T> a{A + row0 * lda, lda, M, tm * BM};
     OperandView<T> b{B + row0 * ldb, ldb, N, tn * BN};
     TG* g = G + (int64_t)e * g_expert_stride;
-    gemm_tile<T, TG, BM, BN, true, true>(a, b, g, g, ldg, ldg, M, N, rows, 0, alpha, beta, smem);
+    gemm_tile2<T, TG, BM, BN, WAVES_M, WAVES_N, true, true>(a, b, g, g, ldg, ldg, M, N, rows, alpha, beta, smem);
 }
 
 static inline int cdiv_i(int64_t a, int b) { return (int)((a + b - 1) / b); }
@@ -139,15 +139,24 @@ extern "C" int fx_grouped_gemm_rows(const void* A, int64_t lda, const void* B, i
     grouped_plan_kernel<<<1, 256, 0, stream>>>(counts, E, BM, w.ntiles, w.offsets, w.tiles);
     FX_CHECK_LAUNCH("fx_grouped_gemm_rows(plan)");
     const unsigned max_tiles = (unsigned)(total_rows / BM + E);
-#define FX_ROWS(TT, BM_, BN_, BMN)                                                                        \
-    grouped_rows_kernel<TT, BM_, BN_, BMN><<<dim3(max_tiles, (unsigned)cdiv_i(N, BN_)), GEMM_THREADS,     \
-                                            (size_t)(BM_ + BN_) * GEMM_BK * sizeof(TT), stream>>>(         \
-        reinterpret_cast<const TT*>(A), lda, reinterpret_cast<const TT*>(B), ldb, b_expert_stride,        \
-        reinterpret_cast<const TT*>(C), ldc, reinterpret_cast<TT*>(D), ldd, w.ntiles, w.offsets, w.tiles, N, K, \
-        alpha, beta)
+#define FX_ROWS(TT, BM_, BN_, WM_, WN_, BMN)                                                              \
+    {                                                                                                     \
+        auto kern = grouped_rows_kernel<TT, BM_, BN_, WM_, WN_, BMN>;                                     \
+        constexpr size_t lds = gemm2_lds_bytes<TT, BM_, BN_, WM_, WN_>();                                 \
+        static bool attr_set = false;                                                                     \
+        if (!attr_set) {                                                                                  \
+            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                \
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);              \
+            attr_set = true;                                                                              \
+        }                                                                                                 \
+        kern<<<dim3(max_tiles, (unsigned)cdiv_i(N, BN_)), WM_ * WN_ * 64, lds, stream>>>(                 \
+            reinterpret_cast<const TT*>(A), lda, reinterpret_cast<const TT*>(B), ldb, b_expert_stride,    \
+            reinterpret_cast<const TT*>(C), ldc, reinterpret_cast<TT*>(D), ldd, w.ntiles, w.offsets,      \
+            w.tiles, N, K, alpha, beta);                                                                  \
+    }
 #define FX_ROWS_T(TT)                                                                                     \
-    if (BM == 256) { if (trans_b) FX_ROWS(TT, 256, 256, false); else FX_ROWS(TT, 256, 256, true); }      \
-    else { if (trans_b) FX_ROWS(TT, 128, 256, false); else FX_ROWS(TT, 128, 256, true); }
+    if (BM == 256) { if (trans_b) FX_ROWS(TT, 256, 256, 4, 2, false) else FX_ROWS(TT, 256, 256, 4, 2, true) } \
+    else { if (trans_b) FX_ROWS(TT, 128, 256, 2, 2, false) else FX_ROWS(TT, 128, 256, 2, 2, true) }
     if (dt == DT_BF16) { FX_ROWS_T(bf16) } else { FX_ROWS_T(f16) }
 #undef FX_ROWS_T
 #undef FX_ROWS
@@ -172,14 +181,23 @@ extern "C" int fx_grouped_gemm_wgrad(const void* A, int64_t lda, const void* B, 
     constexpr int BM = 256, BN = 256;
     const int tiles_m = cdiv_i(M, BM), tiles_n = cdiv_i(N, BN);
     const dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)E);
-    const size_t lds = (size_t)(BM + BN) * GEMM_BK * 2;
 #define FX_WG(TT, TG)                                                                                     \
-    grouped_wgrad_kernel<TT, TG, BM, BN><<<grid, GEMM_THREADS, lds, stream>>>(                            \
-        reinterpret_cast<const TT*>(A), lda, reinterpret_cast<const TT*>(B), ldb, reinterpret_cast<TG*>(G), ldg, \
-        g_expert_stride, w.offsets, M, N, alpha, beta, tiles_n)
-    if (dt == DT_BF16 && g_dt == DT_BF16) FX_WG(bf16, bf16);
-    else if (dt == DT_BF16) FX_WG(bf16, float);
-    else FX_WG(f16, f16);
+    {                                                                                                     \
+        auto kern = grouped_wgrad_kernel<TT, TG, BM, BN, 2, 4>;                                           \
+        constexpr size_t lds = gemm2_lds_bytes<TT, BM, BN, 2, 4>();                                       \
+        static bool attr_set = false;                                                                     \
+        if (!attr_set) {                                                                                  \
+            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                \
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);              \
+            attr_set = true;                                                                              \
+        }                                                                                                 \
+        kern<<<grid, 2 * 4 * 64, lds, stream>>>(reinterpret_cast<const TT*>(A), lda,                      \
+                                                reinterpret_cast<const TT*>(B), ldb, reinterpret_cast<TG*>(G), \
+                                                ldg, g_expert_stride, w.offsets, M, N, alpha, beta, tiles_n); \
+    }
+    if (dt == DT_BF16 && g_dt == DT_BF16) FX_WG(bf16, bf16)
+    else if (dt == DT_BF16) FX_WG(bf16, float)
+    else FX_WG(f16, f16)
 #undef FX_WG
     FX_CHECK_LAUNCH("fx_grouped_gemm_wgrad");
     return 0;

@@ -4,9 +4,10 @@ package (helpers/matmul_dispatcher/matmul_dispatcher/__init__.py:63-276):
 tensors, fp32 accumulation, explicit stream pointer.
 
 ``CublasLtDispatcher`` is kept as the class name callers import; it drives the
-hand-written MFMA GEMM of libflexhip.so through ``dispatch_matmul``.  No
-workspace is allocated (the kernel needs none), and nothing touches the GPU at
-import or construction time.
+hand-written MFMA GEMM of libflexhip.so through ``dispatch_matmul``.  The 64 MiB
+workspace of the reference class is kept (split-K partial sums live there) but is
+allocated on the first call, so nothing touches the GPU at import or construction
+time.
 """
 from __future__ import annotations
 
@@ -70,8 +71,8 @@ class CublasLtDispatcher:
         self.max_algos = max_algos
         self._lib = lib()
         self.ctx = self._lib.create_dispatcher(round_multiple, max_algos)
-        self.workspace_size = 0
-        self.workspace = None
+        self.workspace_size = 64 * 1024 * 1024
+        self.workspace = None           # allocated on first use, on the device of the first operand
         self.ws_ptr = 0
         self.fp16 = torch.float16
         self.bf16 = torch.bfloat16
@@ -82,6 +83,11 @@ class CublasLtDispatcher:
         if getattr(self, "ctx", None):
             self._lib.destroy_dispatcher(self.ctx)
             self.ctx = None
+
+    def _ensure_workspace(self, device):
+        if self.workspace is None or self.workspace.device != device:
+            self.workspace = torch.empty(self.workspace_size, dtype=torch.uint8, device=device)
+            self.ws_ptr = self.workspace.data_ptr()
 
     def get_stats(self):
         stats = (ctypes.c_uint64 * 7)()
@@ -125,6 +131,7 @@ class CublasLtDispatcher:
             raise ValueError(f"All dimensions must be non-zero. Got M={M}, N={N}, K={K}")
         dt = 1 if A.dtype == self.fp16 else (2 if A.dtype == self.bf16 else 0)
         d_dt = _dtype_to_enum.get(D.dtype, dt)
+        self._ensure_workspace(A.device)
         ret = self._lib.dispatch_matmul(self.ctx, stream_ptr, M, N, K, ptr_A, ld_A, ptr_B, ld_B, ptr_C, ld_C,
                                         ptr_D, ld_D, self.ws_ptr, self.workspace_size, dt, dt, d_dt, d_dt, 0,
                                         alpha, beta, trans_a, trans_b)
@@ -155,6 +162,8 @@ class CublasLtDispatcher:
         _, N = B.shape
         dt = _dtype_to_enum[A.dtype]
         d_dt = _dtype_to_enum[D.dtype]
+        if self.workspace is None:
+            self._ensure_workspace(A.device)
         matmul_fast(self._ctx_int, stream_ptr, M, N, K, ptr_A, ld_A, trans_a, ptr_B, ld_B, trans_b, ptr_C, ld_C,
                     ptr_D, ld_D, self.ws_ptr, self.workspace_size, dt, dt, d_dt, d_dt, 0, alpha, beta)
         return D

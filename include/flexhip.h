@@ -243,8 +243,10 @@ int fx_grouped_gemm_wgrad(const void* A, int64_t lda, const void* B, int64_t ldb
  * stride lda; trans_a = 1: A is stored (K,M) with row stride lda.  trans_b = 0:
  * B is (K,N) with row stride ldb; trans_b = 1: B is stored (N,K).  C may be 0
  * (treated as beta = 0) and may alias D.  M, N or K == 0 returns 0 without
- * doing anything.  The workspace arguments are accepted and unused.  A context
- * is not thread-safe; use one per stream, as the reference does. */
+ * doing anything.  The workspace (device memory, 16-byte aligned; the reference
+ * lends cuBLASLt 64 MiB) is used for fp32 partial sums when a problem with few
+ * output tiles and a long K is split along K; without one such problems run
+ * unsplit.  A context is not thread-safe; use one per stream, as the reference does. */
 typedef struct DispatchContext DispatchContext;
 DispatchContext* create_dispatcher(int round_multiple, int max_algos);
 void destroy_dispatcher(DispatchContext* ctx);

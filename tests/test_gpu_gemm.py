@@ -103,3 +103,27 @@ def test_cache_statistics_and_noop(dev):
         disp.matmul(s, A, torch.ones(32, 64, dtype=torch.bfloat16, device=dev))
     with pytest.raises(ValueError):
         tensor_layout(torch.ones(8, 8, 2, device=dev)[:, :, 0])
+
+
+@pytest.mark.parametrize("M,N,K,ta,tb", [(256, 512, 16384, 0, 0), (300, 520, 8200, 0, 1), (1024, 4096, 32064, 0, 0),
+                                         (512, 256, 12288, 1, 0)])
+def test_long_k_few_tiles_splits_along_k(dev, M, N, K, ta, tb):
+    """Few output tiles and a long K: the dispatcher cuts K into ranges, keeps fp32 partial sums in
+    its workspace and reduces them (alpha / beta / C applied once, in the reduction)."""
+    g = gen(M + K)
+    A, B, C = randn(g, M, K, std=0.25), randn(g, K, N, std=0.25), randn(g, M, N)
+    Ad = A.t().contiguous().to(dev).t() if ta else A.to(dev)
+    Bd = B.t().contiguous().to(dev).t() if tb else B.to(dev)
+    disp = CublasLtDispatcher()
+    s = torch.cuda.current_stream().cuda_stream
+    D = disp.matmul(s, Ad, Bd)
+    assert disp.workspace is not None and disp.workspace.numel() == 64 * 1024 * 1024
+    _check(D, _ref(A, B), torch.bfloat16)
+    Cd = C.to(dev)
+    disp.matmul(s, Ad, Bd, C=Cd, D=Cd, alpha=0.5, beta=1.0)
+    _check(Cd, _ref(A, B, C, 0.5, 1.0), torch.bfloat16)
+    # the same shape without a workspace runs unsplit and agrees
+    rc_ws, disp.ws_ptr, disp.workspace_size = disp.ws_ptr, 0, 0
+    D2 = torch.empty_like(D)
+    disp.matmul_fast(s, Ad, Bd, D=D2)
+    _check(D2, _ref(A, B), torch.bfloat16)
