@@ -4,21 +4,22 @@
 //
 // A workgroup of WAVES_M x WAVES_N waves owns a BM x BN tile of D and walks K in steps of
 // 64.  Each wave owns a (BM/WAVES_M) x (BN/WAVES_N) sub-tile built from
-// v_mfma_f32_32x32x16.  Operand tiles live in LDS "K-contiguous": row r (an m or n index)
-// holds its 64 k-values as eight 16-byte chunks, chunk c stored at position c ^ (r & 7).
-// Two LDS buffers alternate, so a K-step needs one barrier: while the matrix pipe works on
-// buffer t, the loads of step t+1 fill buffer t+1.
-//
-// Operands reach LDS in one of two ways:
-//   K-contiguous in memory (A not transposed, B transposed): global_load_lds_dwordx4 moves
-//     16 bytes per lane straight from global memory into LDS, no registers in between; the
-//     XOR swizzle is applied to the global address (a lane picks the chunk that belongs at
-//     its fixed LDS position).
-//   M/N-contiguous in memory (A transposed, B not transposed): a lane loads an 8(k) x 8(mn)
-//     block as eight 16-byte rows, transposes it in registers with v_perm_b32 and writes
-//     eight K-contiguous chunks with ds_write_b128.
-// Rows outside the matrix are clamped to the last valid row (their products are never
-// stored); a K tail shorter than 64 goes through the register path, which zero-fills.
+// v_mfma_f32_32x32x16.  Two LDS buffers alternate, so a K-step needs one barrier: while the
+// matrix pipe works on buffer t, the loads of step t+1 fill buffer t+1.  Both operand forms go
+// from global memory straight into LDS with global_load_lds_dwordx4 (16 bytes per lane, no
+// registers in between); a wave instruction fills 1024 contiguous LDS bytes, so the swizzle is
+// applied to the global address (a lane fetches the chunk that belongs at its fixed LDS place).
+//   K-contiguous in memory (A not transposed, B transposed): LDS row r (an m or n index) holds
+//     its 64 k-values as eight 16-byte chunks, chunk c at position c ^ ((r >> 1) & 7); fragments
+//     are read with ds_read_b128.  The LDS has 64 banks and serves 16 lanes of a b128 read per
+//     cycle: with this swizzle 16 consecutive rows hit 64 distinct banks.
+//   M/N-contiguous in memory (A transposed, B not transposed): LDS row k holds the tile's m (or
+//     n) values, 16-byte chunk c at position c ^ ((k & 3) << 2); fragments are read with
+//     ds_read_b64_tr_b16, which hands lane i of a 16-lane group the i-th element of four rows
+//     (source lanes 4j .. 4j+3 give the address of row j): two reads make the 8 consecutive
+//     k-values of one m that the MFMA wants, without any transposition in registers.
+// Rows / columns outside the matrix are clamped to the last valid ones (their products are
+// never stored); a K tail shorter than 64 goes through registers, which zero-fills.
 #pragma once
 #include "gemm_core.h"
 
@@ -52,6 +53,28 @@ FX_DEV void tile_load_direct(const OperandView<T>& op, int k0, T* lds, int wave,
         g = g < op.ext ? g : op.ext - 1;
         const int c = pos ^ swz(r);
         load_to_lds16(op.base + (int64_t)g * op.ld + k0 + c * 8, lds + (j * NW + wave) * 8 * GEMM_BK);
+    }
+}
+
+// Direct copy of a 64(k) x ROWS M/N-contiguous tile: LDS row k holds ROWS elements, its 16-byte
+// chunk c at position c ^ ((k & 3) << 2).  One wave instruction covers 1024 / (2*ROWS) k-rows.
+FX_DEV int swz_tr(int k) { return (k & 3) << 2; }
+
+template <typename T, int ROWS, int NW>
+FX_DEV void tile_load_direct_tr(const OperandView<T>& op, int k0, T* lds, int wave, int lane) {
+    constexpr int NI = ROWS / 8 / NW;           // instructions per wave: ROWS * 128 bytes in all
+    constexpr int CPR = ROWS / 8;               // 16-byte chunks per LDS row
+    constexpr int KPI = 64 / CPR;               // k-rows per instruction
+    static_assert(ROWS % (8 * NW) == 0 && (ROWS == 64 || ROWS == 128 || ROWS == 256), "unsupported tile rows");
+    const int kin = lane / CPR, pos = lane % CPR;
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+        const int q = j * NW + wave;
+        const int k = q * KPI + kin;
+        const int c = pos ^ (swz_tr(k) % CPR);
+        int g = op.origin + c * 8;
+        g = g + 8 <= op.ext ? g : op.ext - 8;
+        load_to_lds16(op.base + (int64_t)(k0 + k) * op.ld + g, lds + q * 512);
     }
 }
 
@@ -133,56 +156,57 @@ FX_DEV void stage2_store(const Staged2<ROWS, NT>& st, T* lds, int tid) {
     }
 }
 
-// MFMAs of one 64-wide K-step from LDS tiles As (BM rows) and Bs (BN rows).  The fragments
-// of sub-step ks+1 are read from LDS while the MFMAs of sub-step ks run; scheduling
-// barriers pin that order, because left alone the scheduler sinks every read to just
+// MFMAs of one 64-wide K-step from LDS tiles As (BM rows or, when A_TR, 64 k-rows of BM) and Bs.
+// The fragments of sub-step ks+1 are read from LDS while the MFMAs of sub-step ks run;
+// scheduling barriers pin that order, because left alone the scheduler sinks every read to just
 // before its first use and the matrix pipe idles for the LDS latency.
-template <typename T, int WM, int WN>
+template <typename T, int BM, int BN, int WM, int WN, bool A_TR, bool B_TR>
 FX_DEV void mma_step(const T* As, const T* Bs, int row_a0, int row_b0, int lane,
                      f32x16_t (&acc)[WM / 32][WN / 32]) {
     constexpr int TM = WM / 32, TN = WN / 32;
     constexpr int KS = GEMM_BK / 16;
     typedef typename Mfma32<T>::frag frag;
+    typedef short s16x4_t __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) s16x4_t* lds_s16x4_ptr;
     frag af[2][TM], bfv[2][TN];
-    const T* pa[TM];
-    const T* pb[TN];
-    int sa[TM], sb[TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-        const int r = row_a0 + i * 32 + (lane & 31);
-        pa[i] = As + r * GEMM_BK;
-        sa[i] = swz(r);
-    }
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-        const int r = row_b0 + j * 32 + (lane & 31);
-        pb[j] = Bs + r * GEMM_BK;
-        sb[j] = swz(r);
-    }
+    // K-contiguous operand: lane reads row (lane & 31), chunk 2*ks + lane/32.
+    // Transposed-read operand: lane s of 16-lane group g gives the address of row k = 16*ks + 8*(g/2) + s/4
+    // (+4 for the second read), elements 32*i + 16*(g%2) + 4*(s%4) .. +3.
     const int half = lane >> 5;
+    const int grp = lane >> 4, sl = lane & 15;
+    auto read_k = [&](const T* base, int row0, int ks) {
+        const int r = row0 + (lane & 31);
+        return *reinterpret_cast<const frag*>(base + r * GEMM_BK + (((ks * 2 + half) ^ swz(r)) << 3));
+    };
+    auto read_tr = [&](const T* base, int pitch, int col0, int ks) {
+        const int n = col0 + 16 * (grp & 1) + 4 * (sl & 3);
+        const int k = 16 * ks + 8 * (grp >> 1) + (sl >> 2);       // k & 3 is the same for k and k + 4
+        const int off = (((n >> 3) ^ (swz_tr(k) % (pitch / 8))) << 3) + (n & 7);
+        const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(base + k * pitch + off));
+        const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(base + (k + 4) * pitch + off));
+        typedef short s16x8_t __attribute__((ext_vector_type(8)));
+        const s16x8_t both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        return __builtin_bit_cast(frag, both);
+    };
     // read r of sub-step ks: r < TM is A fragment r, otherwise B fragment r - TM
     auto fetch_one = [&](int ks, int slot, int r) {
-        const int chunk = ks * 2 + half;
-        if (r < TM) af[slot][r] = *reinterpret_cast<const frag*>(pa[r] + ((chunk ^ sa[r]) << 3));
-        else bfv[slot][r - TM] = *reinterpret_cast<const frag*>(pb[r - TM] + ((chunk ^ sb[r - TM]) << 3));
+        if (r < TM) af[slot][r] = A_TR ? read_tr(As, BM, row_a0 + r * 32, ks) : read_k(As, row_a0 + r * 32, ks);
+        else bfv[slot][r - TM] = B_TR ? read_tr(Bs, BN, row_b0 + (r - TM) * 32, ks) : read_k(Bs, row_b0 + (r - TM) * 32, ks);
     };
     constexpr int READS = TM + TN, MFMAS = TM * TN;
-    constexpr int EVERY = 1;   // one LDS read after each of the first READS MFMAs
 #pragma unroll
     for (int r = 0; r < READS; ++r) fetch_one(0, 0, r);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
         const int cur = ks & 1;
-        int r = 0;
 #pragma unroll
         for (int m = 0; m < MFMAS; ++m) {
             const int i = m / TN, j = m % TN;
             __builtin_amdgcn_sched_barrier(0);
             acc[i][j] = Mfma32<T>::run(bfv[cur][j], af[cur][i], acc[i][j]);   // transposed tile: rows = n, columns = m
-            if (ks + 1 < KS && m % EVERY == 0 && r < READS) {
+            if (ks + 1 < KS && m < READS) {
                 __builtin_amdgcn_sched_barrier(0);
-                fetch_one(ks + 1, cur ^ 1, r);   // issues in the shadow of the MFMA above
-                ++r;
+                fetch_one(ks + 1, cur ^ 1, m);   // issues in the shadow of the MFMA above
             }
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -282,42 +306,31 @@ FX_DEV void gemm_tile2(const OperandView<T>& A, const OperandView<T>& B, const T
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
     const int nfull = K / GEMM_BK;  // K-steps that need no zero fill
-    Staged2<BM, NT> sa;
-    Staged2<BN, NT> sb;
-
-    // Main loop over the full K-steps: K-contiguous operands go global -> LDS directly,
-    // M/N-contiguous ones through registers (loaded before the MFMAs, written after them).
     auto issue = [&](int kt, T* buf) {
         if (!A_MN) tile_load_direct<T, BM, NW>(A, kt * GEMM_BK, buf, wave, lane);
-        else stage2_load<T, BM, NT, true>(sa, A, kt * GEMM_BK, K, tid);
+        else tile_load_direct_tr<T, BM, NW>(A, kt * GEMM_BK, buf, wave, lane);
         if (!B_MN) tile_load_direct<T, BN, NW>(B, kt * GEMM_BK, buf + BM * GEMM_BK, wave, lane);
-        else stage2_load<T, BN, NT, true>(sb, B, kt * GEMM_BK, K, tid);
+        else tile_load_direct_tr<T, BN, NW>(B, kt * GEMM_BK, buf + BM * GEMM_BK, wave, lane);
     };
-    auto commit = [&](T* buf) {
-        if (A_MN) stage2_store<T, BM, NT, true>(sa, buf, tid);
-        if (B_MN) stage2_store<T, BN, NT, true>(sb, buf + BM * GEMM_BK, tid);
-    };
-    if (nfull > 0) {
-        issue(0, smem);
-        commit(smem);
-    }
+    if (nfull > 0) issue(0, smem);
     for (int kt = 0; kt < nfull; ++kt) {
         T* cur = smem + (kt & 1) * BUF;
         T* nxt = smem + ((kt + 1) & 1) * BUF;
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's direct loads of step kt have landed
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's loads of step kt have landed
         __syncthreads();                                  // everyone's have, and buffer `nxt` is no longer read
         if (kt + 1 < nfull) issue(kt + 1, nxt);
-        mma_step<T, WM, WN>(cur, cur + BM * GEMM_BK, wm * WM, wn * WN, lane, acc);
-        if (kt + 1 < nfull) commit(nxt);
+        mma_step<T, BM, BN, WM, WN, A_MN, B_MN>(cur, cur + BM * GEMM_BK, wm * WM, wn * WN, lane, acc);
     }
-    if (nfull * GEMM_BK < K) {  // K tail: register path for both operands, zero-filled past K
+    if (nfull * GEMM_BK < K) {  // K tail: through registers into the K-contiguous layout, zero-filled past K
+        Staged2<BM, NT> sa;
+        Staged2<BN, NT> sb;
         T* buf = smem + (nfull & 1) * BUF;
         stage2_load<T, BM, NT, A_MN>(sa, A, nfull * GEMM_BK, K, tid);
         stage2_load<T, BN, NT, B_MN>(sb, B, nfull * GEMM_BK, K, tid);
         stage2_store<T, BM, NT, A_MN>(sa, buf, tid);     // `buf` was last read two steps ago
         stage2_store<T, BN, NT, B_MN>(sb, buf + BM * GEMM_BK, tid);
         __syncthreads();
-        mma_step<T, WM, WN>(buf, buf + BM * GEMM_BK, wm * WM, wn * WN, lane, acc);
+        mma_step<T, BM, BN, WM, WN, false, false>(buf, buf + BM * GEMM_BK, wm * WM, wn * WN, lane, acc);
     }
     __syncthreads();  // every wave is past its last LDS read: the buffers become epilogue staging
     static_assert(gemm2_lds_bytes<T, BM, BN, WAVES_M, WAVES_N>() <= 160 * 1024, "tile configuration exceeds the 160 KB of LDS");

@@ -155,7 +155,7 @@ extern "C" int fx_grouped_gemm_rows(const void* A, int64_t lda, const void* B, i
             w.tiles, N, K, alpha, beta);                                                                  \
     }
 #define FX_ROWS_T(TT)                                                                                     \
-    if (BM == 256) { if (trans_b) FX_ROWS(TT, 256, 256, 4, 2, false) else FX_ROWS(TT, 256, 256, 4, 2, true) } \
+    if (BM == 256) { if (trans_b) FX_ROWS(TT, 256, 256, 2, 4, false) else FX_ROWS(TT, 256, 256, 2, 4, true) } \
     else { if (trans_b) FX_ROWS(TT, 128, 256, 2, 2, false) else FX_ROWS(TT, 128, 256, 2, 2, true) }
     if (dt == DT_BF16) { FX_ROWS_T(bf16) } else { FX_ROWS_T(f16) }
 #undef FX_ROWS_T
