@@ -68,22 +68,37 @@ __global__ __launch_bounds__(256) void grouped_plan_kernel(const int32_t* __rest
     if (threadIdx.x == 0) { OFFSETS[E] = carry_r; NTILES[0] = carry_t; }
 }
 
+// pid -> position in the logical order: XCD x (= pid % 8) walks positions [x*per, (x+1)*per).
+FX_DEV int xcd_band(int pid, int total) {
+    constexpr int XCDS = 8;
+    if (total < XCDS * 4) return pid;
+    const int per = total / XCDS, body = per * XCDS;
+    return pid < body ? (pid % XCDS) * per + pid / XCDS : pid;
+}
+
 template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool B_MN>
 __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void grouped_rows_kernel(
     const T* __restrict__ A, int64_t lda, const T* __restrict__ B, int64_t ldb, int64_t b_expert_stride,
     const T* C, int64_t ldc, T* D, int64_t ldd, const int32_t* __restrict__ NTILES,
     const int32_t* __restrict__ OFFSETS, const int32_t* __restrict__ TILES, int N, int K, float alpha,
-    float beta) {
+    float beta, int tiles_n) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T* smem = reinterpret_cast<T*>(smem_raw);
-    const int tile = blockIdx.x;
-    if (tile >= NTILES[0]) return;  // the grid is sized for the worst case
+    // The grid is sized for the worst case; the live tiles are (row tile, column tile) pairs in
+    // expert-major order with the column tile fastest.  Workgroups are dealt round-robin to the 8
+    // XCDs: give each XCD a contiguous band of that order, so the workgroups that share an expert's
+    // weights and a row tile's activations meet in one L2.
+    const int total = NTILES[0] * tiles_n;
+    const int pid = blockIdx.x;
+    if (pid >= total) return;
+    const int p = xcd_band(pid, total);
+    const int tile = p / tiles_n, tn = p % tiles_n;
     const int e = TILES[2 * tile];
     const int m0 = TILES[2 * tile + 1];
     const int64_t row0 = OFFSETS[e];
     const int rows = OFFSETS[e + 1] - OFFSETS[e];
     OperandView<T> a{A + row0 * lda, lda, rows, m0};
-    OperandView<T> b{B + (int64_t)e * b_expert_stride, ldb, N, (int)blockIdx.y * BN};
+    OperandView<T> b{B + (int64_t)e * b_expert_stride, ldb, N, tn * BN};
     const T* c = C ? C + row0 * ldc : nullptr;
     gemm_tile2<T, T, BM, BN, WAVES_M, WAVES_N, false, B_MN>(a, b, c, D + row0 * ldd, ldc, ldd, rows, N, K, alpha, beta, smem);
 }
@@ -92,14 +107,16 @@ template <typename T, typename TG, int BM, int BN, int WAVES_M, int WAVES_N>
 __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void grouped_wgrad_kernel(
     const T* __restrict__ A, int64_t lda, const T* __restrict__ B, int64_t ldb, TG* G, int64_t ldg,
     int64_t g_expert_stride, const int32_t* __restrict__ OFFSETS, int M, int N, float alpha, float beta,
-    int tiles_n) {
+    int tiles_n, int tiles_per_expert) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T* smem = reinterpret_cast<T*>(smem_raw);
-    const int e = blockIdx.y;
+    // expert-major tile order, one contiguous band of it per XCD (see grouped_rows_kernel)
+    const int p = xcd_band(blockIdx.x, gridDim.x);
+    const int e = p / tiles_per_expert, t = p % tiles_per_expert;
     const int64_t row0 = OFFSETS[e];
     const int rows = OFFSETS[e + 1] - OFFSETS[e];
     if (rows == 0 && beta == 1.f) return;  // nothing to add
-    const int tm = blockIdx.x / tiles_n, tn = blockIdx.x % tiles_n;
+    const int tm = t / tiles_n, tn = t % tiles_n;
     OperandView<T> a{A + row0 * lda, lda, M, tm * BM};
     OperandView<T> b{B + row0 * ldb, ldb, N, tn * BN};
     TG* g = G + (int64_t)e * g_expert_stride;
@@ -149,10 +166,11 @@ extern "C" int fx_grouped_gemm_rows(const void* A, int64_t lda, const void* B, i
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);              \
             attr_set = true;                                                                              \
         }                                                                                                 \
-        kern<<<dim3(max_tiles, (unsigned)cdiv_i(N, BN_)), WM_ * WN_ * 64, lds, stream>>>(                 \
+        const int tiles_n = cdiv_i(N, BN_);                                                               \
+        kern<<<dim3(max_tiles * (unsigned)tiles_n), WM_ * WN_ * 64, lds, stream>>>(                       \
             reinterpret_cast<const TT*>(A), lda, reinterpret_cast<const TT*>(B), ldb, b_expert_stride,    \
             reinterpret_cast<const TT*>(C), ldc, reinterpret_cast<TT*>(D), ldd, w.ntiles, w.offsets,      \
-            w.tiles, N, K, alpha, beta);                                                                  \
+            w.tiles, N, K, alpha, beta, tiles_n);                                                         \
     }
 #define FX_ROWS_T(TT)                                                                                     \
     if (BM == 256) { if (trans_b) FX_ROWS(TT, 256, 256, 2, 4, false) else FX_ROWS(TT, 256, 256, 2, 4, true) } \
@@ -180,7 +198,7 @@ extern "C" int fx_grouped_gemm_wgrad(const void* A, int64_t lda, const void* B, 
     FX_CHECK_LAUNCH("fx_grouped_gemm_wgrad(plan)");
     constexpr int BM = 256, BN = 256;
     const int tiles_m = cdiv_i(M, BM), tiles_n = cdiv_i(N, BN);
-    const dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)E);
+    const dim3 grid((unsigned)(tiles_m * tiles_n) * (unsigned)E);
 #define FX_WG(TT, TG)                                                                                     \
     {                                                                                                     \
         auto kern = grouped_wgrad_kernel<TT, TG, BM, BN, 2, 4>;                                           \
@@ -193,7 +211,7 @@ extern "C" int fx_grouped_gemm_wgrad(const void* A, int64_t lda, const void* B, 
         }                                                                                                 \
         kern<<<grid, 2 * 4 * 64, lds, stream>>>(reinterpret_cast<const TT*>(A), lda,                      \
                                                 reinterpret_cast<const TT*>(B), ldb, reinterpret_cast<TG*>(G), \
-                                                ldg, g_expert_stride, w.offsets, M, N, alpha, beta, tiles_n); \
+                                                ldg, g_expert_stride, w.offsets, M, N, alpha, beta, tiles_n, tiles_m * tiles_n); \
     }
     if (dt == DT_BF16 && g_dt == DT_BF16) FX_WG(bf16, bf16)
     else if (dt == DT_BF16) FX_WG(bf16, float)
