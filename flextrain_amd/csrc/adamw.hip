@@ -30,31 +30,45 @@ FX_DEV void adam_elem(float& p, float g, float& m, float& v, const AdamScalars& 
     p = p - a.lr * (mh / denom);
 }
 
-template <typename TP, typename TG, typename TS, bool COPY, bool NT>
+template <typename TP, typename TG, typename TS, bool COPY, bool NT, int UNROLL, bool NTS>
 __global__ __launch_bounds__(ADAM_THREADS) void adamw_kernel(
     TP* __restrict__ P, const TG* __restrict__ G, TS* __restrict__ M, TS* __restrict__ V,
     bf16* __restrict__ PCOPY, int64_t n, AdamScalars a) {
-    const int64_t off = ((int64_t)blockIdx.x * ADAM_THREADS + threadIdx.x) * 8;
-    if (off + 8 <= n) {
-        float p[8], g[8], m[8], v[8];
-        load_f32<TP, 8, NT>(P + off, p);
-        load_f32<TG, 8, NT>(G + off, g);
-        load_f32<TS, 8, NT>(M + off, m);
-        load_f32<TS, 8, NT>(V + off, v);
+    const int64_t base = (int64_t)blockIdx.x * ADAM_THREADS * 8 * UNROLL;
+    float p[UNROLL][8], g[UNROLL][8], m[UNROLL][8], v[UNROLL][8];
+    bool full[UNROLL];
+    // p, m, v are rewritten in place: plain loads (non-temporal ones halve the rate of such
+    // read-modify-write streams); g is read once and the bf16 copy is written once
 #pragma unroll
-        for (int j = 0; j < 8; ++j) adam_elem(p[j], g[j], m[j], v[j], a);
-        store_f32<TP, 8, NT>(P + off, p);
-        store_f32<TS, 8, NT>(M + off, m);
-        store_f32<TS, 8, NT>(V + off, v);
-        if (COPY) store_f32<bf16, 8, NT>(PCOPY + off, p);
-    } else {
-        for (int64_t i = off; i < n; ++i) {
-            float p = (float)P[i], g = (float)G[i], m = (float)M[i], v = (float)V[i];
-            adam_elem(p, g, m, v, a);
-            P[i] = (TP)p;
-            M[i] = (TS)m;
-            V[i] = (TS)v;
-            if (COPY) PCOPY[i] = (bf16)p;
+    for (int u = 0; u < UNROLL; ++u) {
+        const int64_t off = base + ((int64_t)u * ADAM_THREADS + threadIdx.x) * 8;
+        full[u] = off + 8 <= n;
+        if (full[u]) {
+            load_f32<TP, 8>(P + off, p[u]);
+            load_f32<TG, 8, NT>(G + off, g[u]);
+            load_f32<TS, 8>(M + off, m[u]);
+            load_f32<TS, 8>(V + off, v[u]);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+        const int64_t off = base + ((int64_t)u * ADAM_THREADS + threadIdx.x) * 8;
+        if (full[u]) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) adam_elem(p[u][j], g[u][j], m[u][j], v[u][j], a);
+            store_f32<TP, 8, NTS>(P + off, p[u]);
+            store_f32<TS, 8, NTS>(M + off, m[u]);
+            store_f32<TS, 8, NTS>(V + off, v[u]);
+            if (COPY) store_f32<bf16, 8, NT>(PCOPY + off, p[u]);
+        } else {
+            for (int64_t i = off; i < n && i < off + 8; ++i) {
+                float pp = (float)P[i], gg = (float)G[i], mm = (float)M[i], vv = (float)V[i];
+                adam_elem(pp, gg, mm, vv, a);
+                P[i] = (TP)pp;
+                M[i] = (TS)mm;
+                V[i] = (TS)vv;
+                if (COPY) PCOPY[i] = (bf16)pp;
+            }
         }
     }
 }
@@ -74,17 +88,19 @@ __global__ __launch_bounds__(256) void nonfinite_kernel(const T* __restrict__ X,
 template <typename TP, typename TG, typename TS>
 static void launch_adamw(void* p, const void* g, void* m, void* v, void* pcopy, int64_t n,
                          const AdamScalars& a, hipStream_t s) {
-    const unsigned grid = (unsigned)((n + (int64_t)ADAM_THREADS * 8 - 1) / ((int64_t)ADAM_THREADS * 8));
     TP* P = reinterpret_cast<TP*>(p);
     const TG* G = reinterpret_cast<const TG*>(g);
     TS* M = reinterpret_cast<TS*>(m);
     TS* V = reinterpret_cast<TS*>(v);
     bf16* C = reinterpret_cast<bf16*>(pcopy);
     const bool nt = (size_t)n * (2 * sizeof(TP) + sizeof(TG) + 4 * sizeof(TS)) >= kStreamingBytes;
-    if (pcopy && nt) adamw_kernel<TP, TG, TS, true, true><<<grid, ADAM_THREADS, 0, s>>>(P, G, M, V, C, n, a);
-    else if (pcopy) adamw_kernel<TP, TG, TS, true, false><<<grid, ADAM_THREADS, 0, s>>>(P, G, M, V, C, n, a);
-    else if (nt) adamw_kernel<TP, TG, TS, false, true><<<grid, ADAM_THREADS, 0, s>>>(P, G, M, V, C, n, a);
-    else adamw_kernel<TP, TG, TS, false, false><<<grid, ADAM_THREADS, 0, s>>>(P, G, M, V, C, n, a);
+#define GO(U, NTS_) { const int64_t per = (int64_t)ADAM_THREADS * 8 * U; const unsigned grid = (unsigned)((n + per - 1) / per); \
+    if (pcopy && nt) adamw_kernel<TP, TG, TS, true, true, U, NTS_><<<grid, ADAM_THREADS, 0, s>>>(P, G, M, V, C, n, a); \
+    else if (pcopy) adamw_kernel<TP, TG, TS, true, false, U, NTS_><<<grid, ADAM_THREADS, 0, s>>>(P, G, M, V, C, n, a); \
+    else if (nt) adamw_kernel<TP, TG, TS, false, true, U, NTS_><<<grid, ADAM_THREADS, 0, s>>>(P, G, M, V, C, n, a); \
+    else adamw_kernel<TP, TG, TS, false, false, U, NTS_><<<grid, ADAM_THREADS, 0, s>>>(P, G, M, V, C, n, a); }
+    GO(1, false)
+#undef GO
 }
 
 }  // namespace fx

@@ -279,7 +279,16 @@ __global__ __launch_bounds__(256) void rmsnorm_dw_reduce_kernel(
     const int col = blockIdx.x * 32 + cl;
     float acc = 0.f;
     if (col < ncols) {
-        for (int b = sl; b < nparts; b += 8) acc += PARTIAL[(size_t)b * ncols + col];
+        // eight independent loads in flight per lane; the additions keep their fixed order
+        int b = sl;
+        for (; b + 56 < nparts; b += 64) {
+            float t[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) t[u] = PARTIAL[(size_t)(b + 8 * u) * ncols + col];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) acc += t[u];
+        }
+        for (; b < nparts; b += 8) acc += PARTIAL[(size_t)b * ncols + col];
     }
     sm[sl][cl] = acc;
     __syncthreads();

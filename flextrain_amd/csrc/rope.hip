@@ -68,7 +68,33 @@ __global__ __launch_bounds__(ROPE_THREADS) void rope_vec_kernel(
 #pragma unroll
         for (int j = 0; j < 4; ++j) { c[j] = tcs[(v * 4 + j) * 2]; s[j] = tcs[(v * 4 + j) * 2 + 1]; }
         const int hstep = tpt / vec_per_head;
-        for (int h = lane / vec_per_head; h < Hq + Hk; h += hstep) rotate(h, v, c, s);
+        // four heads per round: all loads are issued before the first store, so a lane has up to
+        // 64 bytes in flight instead of one load -> rotate -> store chain per head
+        for (int h0 = lane / vec_per_head; h0 < Hq + Hk; h0 += 4 * hstep) {
+            float x[4][8];
+            T* ptr[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int h = h0 + u * hstep;
+                ptr[u] = nullptr;
+                if (h < Hq + Hk) {
+                    ptr[u] = ((h < Hq) ? (Q + t * sq_t + (int64_t)h * sq_h) : (K + t * sk_t + (int64_t)(h - Hq) * sk_h)) + v * 8;
+                    load_f32<T, 8, NT>(ptr[u], x[u]);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if (ptr[u] == nullptr) continue;
+                float y[8];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float e = x[u][2 * j], o = x[u][2 * j + 1];
+                    y[2 * j] = e * c[j] - o * s[j];
+                    y[2 * j + 1] = e * s[j] + o * c[j];
+                }
+                store_f32<T, 8, NT>(ptr[u], y);
+            }
+        }
     } else {
         for (int it = lane; it < items; it += tpt) {
             const int h = it / vec_per_head;
@@ -128,7 +154,8 @@ static int launch_rope(void* q, void* k, const int32_t* pos, int64_t stride_pos,
         while (tpb < 16 && items * tpb * 2 <= ROPE_THREADS) tpb *= 2;
         const size_t lds = (size_t)tpb * (rot_dim >> 1) * 2 * sizeof(float);
         const unsigned grid = (unsigned)((T_tokens + tpb - 1) / tpb);
-        const bool nt = (size_t)T_tokens * (Hq + Hk) * rot_dim * sizeof(T) * 2 >= kStreamingBytes;
+        // the rotation is in place: plain accesses (non-temporal ones slow read-modify-write streams down)
+        const bool nt = false;
         if (nt)
             rope_vec_kernel<T, BWD, true><<<grid, ROPE_THREADS, lds, s>>>(
                 Q, K, pos, stride_pos, inv_freq, stride_if, T_tokens, Hq, Hk, D, rot_dim, sq[0], sq[1],
