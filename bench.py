@@ -234,7 +234,10 @@ def run_lm_head(torch, dev, stream, rn):
 
     rows = []
     ms = _time_launches(torch, stream, [run], warmup=1, reps=3)
-    rows.append(_op_entry("c3.lm_head fwd+bwd (chunk 1024, fp32 dW)", 6 * T * d * V, "TFLOP/s", ms))
+    rows.append(_op_entry("c3.lm_head fwd+bwd (chunk 1024 x 8 fused per GEMM group, fp32 dW)", 6 * T * d * V, "TFLOP/s", ms))
+    head = LMHead(LMHeadConfig(d_model=d, vocab_size=V, head_chunk_size=chunk, fuse_chunks=1))
+    ms = _time_launches(torch, stream, [run], warmup=1, reps=3)
+    rows.append(_op_entry("c3.lm_head fwd+bwd (chunk 1024, one GEMM group per chunk as the reference, fp32 dW)", 6 * T * d * V, "TFLOP/s", ms))
     # the three GEMMs of one micro-chunk, timed alone
     disp = CublasLtDispatcher()
     sp = stream.cuda_stream

@@ -2,7 +2,7 @@
 interface of flextrain/nn/head.py:60-393 (``LMHeadConfig``, ``LMHead.forward_backward``)
 and ``LossStats`` (flextrain/core/layer.py:1060-1088).
 
-Per micro-chunk: RMSNorm fwd -> logits GEMM -> loss fn (dZ in place) -> head
+Per group of micro-chunks: RMSNorm fwd -> logits GEMM -> loss fn (dZ in place) -> head
 weight-gradient GEMM (``beta = 1``, ``alpha = loss_scale``) -> dX GEMM -> RMSNorm
 bwd -> dx written over x.  The GEMMs go through the MFMA dispatcher; the
 weight may be stored ``(d_model, vocab)`` (reference) or be the transposed view
@@ -28,6 +28,12 @@ class LMHeadConfig:
     vocab_size: int
     rms_norm_eps: float = 1e-5
     head_chunk_size: int = 1024
+    # Micro-chunks handled by one GEMM group (not in the reference, whose 24-32 GB cards force one
+    # logits buffer of head_chunk_size rows).  None: as many as keep the logits buffer under
+    # ``logits_buffer_bytes``.  Larger groups mean fewer read-modify-write passes over the head
+    # weight gradient and better-filled GEMMs; the result differs only in accumulation order.
+    fuse_chunks: int | None = None
+    logits_buffer_bytes: int = 4 << 30
     final_logit_softcap: float | None = None
     compute_dtype: torch.dtype = torch.bfloat16
     master_dtype: torch.dtype | None = None
@@ -85,13 +91,18 @@ class LMHead:
         disp = self._dispatcher()
         stream = torch.cuda.current_stream(device).cuda_stream
         aux_chunks = []
-        chunk_rows = min(cfg.head_chunk_size, num_tokens)
+        fuse = cfg.fuse_chunks
+        if fuse is None:
+            per_chunk = cfg.head_chunk_size * V * x.element_size()
+            fuse = max(1, cfg.logits_buffer_bytes // max(1, per_chunk))
+        group_rows = cfg.head_chunk_size * max(1, int(fuse))
+        chunk_rows = min(group_rows, num_tokens)
         logits_buf = torch.empty((chunk_rows, V), dtype=dtype, device=device)
         dx_head_buf = torch.empty((chunk_rows, d_model), dtype=dtype, device=device)
 
         offset = 0
         while offset < num_tokens:
-            t_prime = min(cfg.head_chunk_size, num_tokens - offset)
+            t_prime = min(group_rows, num_tokens - offset)
             x_slice = x[offset:offset + t_prime]
             head_in, rstd = flextrain_rmsnorm_fwd(x_slice, W=w_final_norm, rms_norm_eps=cfg.rms_norm_eps)
             logits = logits_buf[:t_prime]

@@ -108,7 +108,8 @@ def _head_inputs(seed, T, d, V, hf_layout):
 
 @pytest.mark.parametrize("hf_layout", [True, False])
 @pytest.mark.parametrize("fused", [True, False])
-def test_lm_head_forward_backward(dev, hf_layout, fused):
+@pytest.mark.parametrize("fuse_chunks", [None, 1, 2])
+def test_lm_head_forward_backward(dev, hf_layout, fused, fuse_chunks):
     T, d, V, chunk = 300, 256, 5000, 128
     x, w_norm, w, labels = _head_inputs(21, T, d, V, hf_layout)
     scale = 1.0 / int((labels != -100).sum())
@@ -118,7 +119,7 @@ def test_lm_head_forward_backward(dev, hf_layout, fused):
     g_store = torch.zeros((V, d) if hf_layout else (d, V), dtype=torch.float32, device=dev)
     g_head = g_store.t() if hf_layout else g_store
     g_norm = torch.zeros(d, dtype=torch.float32, device=dev)
-    head = LMHead(LMHeadConfig(d_model=d, vocab_size=V, head_chunk_size=chunk))
+    head = LMHead(LMHeadConfig(d_model=d, vocab_size=V, head_chunk_size=chunk, fuse_chunks=fuse_chunks))
     xd = x.to(dev)
     dx, stats = head.forward_backward(xd, TokenContext(labels=labels.to(dev)), None,
                                       {"w_final_norm": w_norm.to(dev), "w_head_proj": wd},
