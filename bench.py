@@ -33,6 +33,11 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0       # MI355X HBM3E, published
 BF16_PEAK_TFLOPS = 2500.0    # MI355X dense bf16 MFMA, published
 
+# HBM bytes per launch of the SwiGLU backward kernel at the benchmark shape, from the FETCH_SIZE and
+# WRITE_SIZE hardware counters scaled by what they read for a plain copy of known size
+# (profiles/glu_bwd_hbm_traffic_pmc.txt holds the counter values and the commands).
+GLU_BWD_MEASURED_TRAFFIC_BYTES = 1_174_223_936
+
 METRIC = "per-op HBM GB/s (% of 8 TB/s) + lm_head/MoE GEMM TFLOPS (% bf16 MFMA peak)"
 
 
@@ -148,6 +153,32 @@ def run_extra(torch, ops, dev, stream, rn):
     rows += run_lm_head(torch, dev, stream, rn)
     rows += run_moe(torch, dev, stream, rn)
     return rows
+
+
+def run_mfma_probe(torch, dev, stream):
+    """What the matrix pipes sustain on this machine with nothing else going on: bf16 MFMAs only,
+    operands in registers.  Constant data reaches the published peak; random data makes the power
+    management lower the clock, and that rate is the practical ceiling for a GEMM on real data."""
+    import ctypes
+
+    from flextrain_amd._lib import lib
+
+    L = lib()
+    ws = torch.empty(int(L.fx_probe_ws_bytes()), dtype=torch.uint8, device=dev)
+    out = {}
+    for name, rnd in (("constant_operands", 0), ("random_operands", 1)):
+        flop = ctypes.c_double()
+        iters = 120000      # ~30-40 ms: long enough for the clock to settle under load
+
+        def launch():
+            L.fx_probe_mfma_rate(rnd, iters, ws.data_ptr(), ws.numel(), ctypes.byref(flop), stream.cuda_stream)
+
+        ms = _time_launches(torch, stream, [launch], warmup=1, reps=3)
+        clocks = ws[:16].view(torch.int64).cpu()
+        ghz = float(clocks[0]) / max(1.0, float(clocks[1])) * 0.1      # wall clock ticks at 100 MHz
+        out[name] = {"tflops": round(flop.value / (ms * 1e-3) / 1e12, 1), "shader_clock_ghz": round(ghz, 3),
+                     "ms": round(ms, 3)}
+    return out
 
 
 def run_streamed_adamw(torch, dev):
@@ -384,6 +415,9 @@ def main():
         rec("swiglu_bwd", lambda: ops.flextrain_swiglu_bwd(gate, up, dout, dx1=dgate, dx3=dup))
         rec("rope_bwd", lambda: ops.flextrain_rope_bwd([q, k], pos, inv_freq))
 
+    # one plain copy of known size (reads and writes 234,881,024 bytes each): the yardstick that hardware
+    # counter runs of this script scale FETCH_SIZE / WRITE_SIZE by
+    out.copy_(gate)
     untimed = lambda name, fn: fn()
     with torch.cuda.stream(stream):
         for _ in range(args.warmup):
@@ -404,12 +438,18 @@ def main():
     dom_gbps = swiglu_bwd_bytes / (dom_ms * 1e-3) / 1e9
     roofline = {"kernel": "glu_bwd_kernel<bf16, silu>", "bound": "hbm", "achieved": round(dom_gbps, 1),
                 "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(dom_gbps / HBM_PEAK_GBPS, 4),
-                "traffic": None, "algorithmic_bytes": swiglu_bwd_bytes, "avg_ms": round(dom_ms, 5)}
+                "traffic": GLU_BWD_MEASURED_TRAFFIC_BYTES, "algorithmic_bytes": swiglu_bwd_bytes, "avg_ms": round(dom_ms, 5)}
     del q, k, gate, up, dout, out, dgate, dup
 
     # ------------------------------------------------- other configurations
+    mfma_probe = None
     if not args.no_extra:
         op_rows += run_extra(torch, ops, dev, stream, rn)
+        mfma_probe = run_mfma_probe(torch, dev, stream)
+        for row in op_rows:
+            if row["unit"] == "TFLOP/s":
+                row["frac_of_sustained_mfma_random_operands"] = round(
+                    row["achieved"] / mfma_probe["random_operands"]["tflops"], 4)
 
     # -------------------------------------------------------- CPU baseline
     cpu = None
@@ -465,6 +505,7 @@ def main():
                    "algorithmic_bytes_per_step": step_bytes},
         "roofline": roofline,
         "cpu_baseline": cpu,
+        "mfma_probe": mfma_probe,
         "ops": op_rows,
     }
     print(json.dumps(result))

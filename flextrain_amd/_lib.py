@@ -92,6 +92,8 @@ _SIGNATURES = {
                                       c_int, c_int, c_float, c_float, c_float, c_float, c_float, c_float,
                                       c_float, c_void_p, c_size_t, c_int64, c_int, c_void_p, c_void_p,
                                       c_void_p]),
+    "fx_probe_ws_bytes": (c_size_t, []),
+    "fx_probe_mfma_rate": (c_int, [c_int, c_int, c_void_p, c_size_t, POINTER(c_double), c_void_p]),
     "solve_scheduler": (c_double, [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_double, c_int, c_int,
                                    c_void_p]),
     "compute_buf_size": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p, c_double, c_int]),

@@ -297,6 +297,17 @@ int fx_adamw_stream_chunk(void* p_host, const void* g_host, void* m_host, void* 
                           float bias_correction2, void* ws, size_t ws_bytes, int64_t sub_elems, int n_slots,
                           hipStream_t inbound, hipStream_t compute, hipStream_t outbound);
 
+/* ---- Hardware probe --------------------------------------------------------- */
+
+/* No counterpart in the reference: a benchmark aid.  Launches one workgroup per CU that issues
+ * nothing but bf16 MFMAs (operands in registers; constant data, or random data when random_data
+ * != 0) for `iters` rounds of 16 instructions per wave, on `stream`.  *flop_out receives the
+ * floating-point operations of the launch (the caller times it); the first 16 bytes of ws
+ * (fx_probe_ws_bytes() bytes of device memory) receive two uint64: shader clock cycles and
+ * 100 MHz wall-clock ticks spent in the loop, from which the clock under load follows. */
+size_t fx_probe_ws_bytes(void);
+int fx_probe_mfma_rate(int random_data, int iters, void* ws, size_t ws_bytes, double* flop_out, hipStream_t stream);
+
 /* ---- Save-level transmission scheduler (verbatim ABI of the reference helper) -- */
 
 /* helpers/transmission_scheduler/transmission_scheduler/transmission_scheduler.h:23-36
