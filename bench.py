@@ -48,6 +48,8 @@ def _parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-extra", action="store_true", help="skip the non-headline configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--only", default="", help="comma-separated subset of the non-headline configurations "
+                                               "(c1, c3, c4, c5) to run, e.g. for a profiler pass")
     return ap.parse_args()
 
 
@@ -101,7 +103,22 @@ def _time_launches(torch, stream, fns, warmup=5, reps=20):
     return a.elapsed_time(b) / reps
 
 
-def run_extra(torch, ops, dev, stream, rn):
+def run_extra(torch, ops, dev, stream, rn, only):
+    want = lambda tag: not only or tag in only
+    rows = []
+    if want("c1"):
+        rows += run_rmsnorm(torch, ops, dev, stream, rn)
+    if want("c4"):
+        rows += run_adamw(torch, ops, dev, stream)
+        rows += run_streamed_adamw(torch, dev)
+    if want("c3"):
+        rows += run_lm_head(torch, dev, stream, rn)
+    if want("c5"):
+        rows += run_moe(torch, dev, stream, rn)
+    return rows
+
+
+def run_rmsnorm(torch, ops, dev, stream, rn):
     rows = []
     # ---- configs[0]: RMSNorm fwd+bwd, x [2048,4096] bf16; 24 buffer sets = 1.6 GB
     T, D, NSETS = 2048, 4096, 24
@@ -128,8 +145,12 @@ def run_extra(torch, ops, dev, stream, rn):
     rows.append(_op_entry("c1.rmsnorm_bwd(dX+=,dW+=,y)", 5 * T * D * 2 + D * 2 + T * 4 + 2 * D * 4, "GB/s", ms))
     del sets, fwd, bwd, bwd_e
     torch.cuda.empty_cache()
+    return rows
 
-    # ---- configs[3] kernel: AdamW on one 218,112,000-parameter chunk resident in HBM
+
+def run_adamw(torch, ops, dev, stream):
+    """configs[3] kernel: AdamW on one 218,112,000-parameter chunk resident in HBM."""
+    rows = []
     n = 218_112_000
     p = (torch.randn(n, device=dev) * 0.02)
     m = torch.zeros(n, device=dev)
@@ -149,9 +170,6 @@ def run_extra(torch, ops, dev, stream, rn):
     rows.append(_op_entry("c4.adamw(fp32 p/m/v, bf16 g)", 26 * n, "GB/s", ms))
     del p, m, v, gr, pb
     torch.cuda.empty_cache()
-    rows += run_streamed_adamw(torch, dev)
-    rows += run_lm_head(torch, dev, stream, rn)
-    rows += run_moe(torch, dev, stream, rn)
     return rows
 
 
@@ -444,7 +462,7 @@ def main():
     # ------------------------------------------------- other configurations
     mfma_probe = None
     if not args.no_extra:
-        op_rows += run_extra(torch, ops, dev, stream, rn)
+        op_rows += run_extra(torch, ops, dev, stream, rn, [t.strip() for t in args.only.split(",") if t.strip()])
         mfma_probe = run_mfma_probe(torch, dev, stream)
         for row in op_rows:
             if row["unit"] == "TFLOP/s":
