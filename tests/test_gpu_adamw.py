@@ -65,3 +65,24 @@ def test_errors(dev):
         ops.flextrain_adamw_step(torch.ones(4), torch.ones(4), torch.ones(4), torch.ones(4))
     e = torch.zeros(0, device=dev)
     assert ops.flextrain_adamw_step(e, e, e, e) == 0
+
+
+def test_full_size_offloaded_layer_chunk(dev):
+    """218,112,000 parameters (one Llama-3.1-8B decoder layer), fp32 master weights and moments, bf16
+    gradients, three prior steps, the measured step is step 4, bf16 copy of the new weights; against
+    the CPU oracle on every element (fp32 state: rtol 1e-4, absolute floors as in the test above)."""
+    n = 218_112_000
+    g = gen(1003)
+    p = torch.empty(n).normal_(0, 0.02, generator=g)
+    m = torch.zeros(n)
+    v = torch.zeros(n)
+    pd, md, vd = p.to(dev), m.to(dev), v.to(dev)
+    pb = torch.empty(n, dtype=torch.bfloat16, device=dev)
+    for step in range(1, 5):
+        gr = torch.empty(n).normal_(0, 1e-3, generator=g).to(torch.bfloat16)
+        p, m, v, pbf = o_adamw.adamw_step(p, gr, m, v, step=step, **HP)
+        assert ops.flextrain_adamw_step(pd, gr.to(dev), md, vd, step=step, params_bf16_out=pb, **HP) == 0
+    torch.testing.assert_close(pd.cpu(), p, rtol=1e-4, atol=1e-9)
+    torch.testing.assert_close(md.cpu(), m, rtol=1e-4, atol=1e-8)
+    torch.testing.assert_close(vd.cpu(), v, rtol=1e-4, atol=1e-12)
+    assert torch.equal(pb.cpu(), pd.to(torch.bfloat16).cpu())

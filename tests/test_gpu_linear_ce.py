@@ -9,6 +9,8 @@ from flextrain_amd import ops
 from flextrain_amd.head import LMHead, LMHeadConfig
 from flextrain_amd.loss import CrossEntropyLoss, TokenContext
 from oracle import linear_ce as o_ce
+from oracle.rmsnorm import rmsnorm_bwd as o_norm_bwd
+from oracle.rmsnorm import rmsnorm_fwd as o_norm_fwd
 from util import F32_RTOL, close, gen, randn
 
 pytestmark = pytest.mark.gpu
@@ -160,3 +162,50 @@ def test_lm_head_skips_missing_grads_and_bf16_accumulator(dev):
     with pytest.raises(ValueError):
         head.forward_backward(x.to(dev), TokenContext(labels=labels[:10].to(dev)), None,
                               {"w_final_norm": w_norm.to(dev), "w_head_proj": wd}, {}, None)
+
+
+def test_full_size_llama_head(dev):
+    """hidden [8192,4096], lm_head [128256,4096], 10 % ignored labels, micro-chunk 1024.  The oracle runs
+    on a sample of token rows (whole vocabulary rows of logits, loss, dZ and the row's dx); everything
+    else is checked through properties that hold at any size: the grouped (8 x 1024) and the per-chunk
+    schedules agree, ignored rows have zero loss, and the head gradient sums to ~0 over the vocabulary
+    (every kept row of dZ sums to 0)."""
+    T, d, V, chunk = 8192, 4096, 128256, 1024
+    g = gen(1002)
+    x = randn(g, T, d)
+    w = (torch.empty(V, d).normal_(0, 0.02, generator=g)).to(torch.bfloat16)
+    w_norm = torch.ones(d)
+    labels = torch.randint(0, V, (T,), generator=g)
+    labels[torch.rand(T, generator=g) < 0.1] = -100
+    scale = 1.0 / int((labels != -100).sum())
+    wd, ld, wn = w.to(dev), labels.to(dev), w_norm.to(dev)
+
+    def run(fuse):
+        xd = x.to(dev)
+        gh = torch.zeros(V, d, dtype=torch.float32, device=dev)
+        gn = torch.zeros(d, dtype=torch.float32, device=dev)
+        head = LMHead(LMHeadConfig(d_model=d, vocab_size=V, head_chunk_size=chunk, fuse_chunks=fuse))
+        dx, stats = head.forward_backward(xd, TokenContext(labels=ld), None, {"w_final_norm": wn, "w_head_proj": wd.t()},
+                                          {"g_head_proj": gh.t(), "g_final_norm": gn}, None, loss_scale=scale)
+        return dx, stats, gh, gn
+
+    dx, stats, gh, gn = run(None)
+    dx1, stats1, gh1, gn1 = run(1)
+    # schedule independence (accumulation order differs: bf16 dx, fp32 head gradient)
+    close(stats.per_token_loss, stats1.per_token_loss, rtol=1e-4, atol=1e-4, what="loss grouped vs per chunk")
+    close(dx, dx1, rtol=1e-2, atol=1e-2 * dx1.float().abs().max().item(), what="dx grouped vs per chunk")
+    close(gh, gh1, rtol=1e-2, atol=1e-2 * gh1.abs().max().item(), what="g_head grouped vs per chunk")
+    close(gn, gn1, rtol=1e-2, atol=1e-2 * gn1.abs().max().item(), what="g_norm grouped vs per chunk")
+    loss = stats.per_token_loss.cpu()
+    assert not loss[labels == -100].any() and bool((loss[labels != -100] > 0).all())
+    col = gh.sum(dim=0)                       # sum over the vocabulary of d(loss)/dW[v, :]
+    assert float(col.abs().max()) <= 2e-3 * float(gh.abs().sum(dim=0).max()), "head gradient must sum to ~0 over V"
+    # sampled rows against the oracle
+    rows = torch.cat([torch.arange(0, 8), torch.arange(4090, 4098), torch.tensor([T - 1])])
+    h, rstd = o_norm_fwd(x[rows], w_norm)
+    logits = (h.float() @ w.float().t()).to(torch.bfloat16)
+    dz_ref, loss_ref, _, _ = o_ce.softmax_ce(logits, labels[rows])
+    close(loss[rows], loss_ref, rtol=5e-3, atol=5e-3, what="sampled per-token loss")
+    dh = (scale * (dz_ref.float() @ w.float())).to(torch.bfloat16)
+    dx_ref, _, _ = o_norm_bwd(dh, x[rows], w_norm, rstd)
+    close(dx.cpu()[rows], dx_ref, rtol=2e-2, atol=2e-2 * dx_ref.float().abs().max().item(), what="sampled dx")
