@@ -43,6 +43,9 @@ _SIGNATURES = {
     "fx_glu_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_void_p]),
     "fx_glu_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
                            c_int, c_int, c_void_p]),
+    "fx_silu_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_void_p]),
+    "fx_embedding_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int, c_int64, c_int64,
+                                 c_int64, c_int64, c_int64, c_float, c_int, c_int, c_void_p]),
     "fx_adamw_step": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int,
                               c_int, c_int, c_float, c_float, c_float, c_float, c_float, c_float,
                               c_float, c_void_p]),

@@ -130,6 +130,36 @@ __global__ __launch_bounds__(GLU_THREADS) void glu_bwd_kernel(
     }
 }
 
+// d/dz silu(z) * dout = dout * s * (1 + z * (1 - s)), s = sigmoid(z)  (flextrain/ops/_kernels/silu_bwd.py:16-35).
+template <typename T, bool NT>
+__global__ __launch_bounds__(GLU_THREADS) void silu_bwd_kernel(const T* Z, const T* DOUT, T* DIN /* may alias Z or DOUT */, int64_t n,
+                                                               bool vec) {
+    if (vec) {
+        const int64_t off = ((int64_t)blockIdx.x * GLU_THREADS + threadIdx.x) * 8;
+        if (off + 8 <= n) {
+            float z[8], d[8], o[8];
+            load_f32<T, 8, NT>(Z + off, z);
+            load_f32<T, 8, NT>(DOUT + off, d);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float sg = fast_sigmoid(z[j]);
+                o[j] = d[j] * (sg * (1.0f + z[j] * (1.0f - sg)));
+            }
+            store_f32<T, 8, NT>(DIN + off, o);
+            return;
+        }
+        for (int64_t i = off; i < n; ++i) {
+            const float zz = (float)Z[i], sg = fast_sigmoid(zz);
+            DIN[i] = (T)((float)DOUT[i] * (sg * (1.0f + zz * (1.0f - sg))));
+        }
+    } else {
+        for (int64_t i = ((int64_t)blockIdx.x * GLU_THREADS + threadIdx.x) * 8, e = i + 8; i < n && i < e; ++i) {
+            const float zz = (float)Z[i], sg = fast_sigmoid(zz);
+            DIN[i] = (T)((float)DOUT[i] * (sg * (1.0f + zz * (1.0f - sg))));
+        }
+    }
+}
+
 // Unaligned-pointer fallback: one element per lane.
 template <typename T, typename TO, int ACT>
 __global__ __launch_bounds__(256) void glu_fwd_scalar_kernel(const T* X1, const T* X3, TO* OUT, int64_t n) {
@@ -217,5 +247,20 @@ extern "C" int fx_glu_bwd(const void* x1, const void* x3, const void* dout, void
         if (act == ACT_SILU) launch_glu_bwd<T, ACT_SILU>(x1, x3, dout, dx1, dx3, act_out, n, stream);
         else launch_glu_bwd<T, ACT_GELU_TANH>(x1, x3, dout, dx1, dx3, act_out, n, stream));
     FX_CHECK_LAUNCH("fx_glu_bwd");
+    return 0;
+}
+
+extern "C" int fx_silu_bwd(const void* z, const void* dout, void* din, int64_t n, int dt, hipStream_t stream) {
+    if (n < 0) FX_FAIL("fx_silu_bwd: negative element count");
+    if (n == 0) return 0;
+    if (!z || !dout || !din) FX_FAIL("fx_silu_bwd: null pointer");
+    const bool vec = aligned16(z) && aligned16(dout) && aligned16(din);
+    const unsigned grid = (unsigned)((n + (int64_t)GLU_THREADS * 8 - 1) / ((int64_t)GLU_THREADS * 8));
+    FX_DISPATCH_DTYPE(dt, T,
+        if ((size_t)n * 3 * sizeof(T) >= kStreamingBytes && din != z && din != dout)
+            silu_bwd_kernel<T, true><<<grid, GLU_THREADS, 0, stream>>>(reinterpret_cast<const T*>(z), reinterpret_cast<const T*>(dout), reinterpret_cast<T*>(din), n, vec);
+        else
+            silu_bwd_kernel<T, false><<<grid, GLU_THREADS, 0, stream>>>(reinterpret_cast<const T*>(z), reinterpret_cast<const T*>(dout), reinterpret_cast<T*>(din), n, vec));
+    FX_CHECK_LAUNCH("fx_silu_bwd");
     return 0;
 }

@@ -9,6 +9,7 @@ from .glu import (
     flextrain_swiglu_bwd,
     flextrain_swiglu_fwd,
 )
+from .misc import flextrain_embedding_bwd, flextrain_silu_bwd
 from .moe import (
     flextrain_copy_expert_counts,
     flextrain_fused_topk_softmax,
@@ -40,8 +41,31 @@ from .rope import (
     flextrain_rope_partial_fwd,
 )
 
+from ..host_memory import destroy_pinned_tensor, pin_tensor
+
+_dispatchers = {}
+
+
+def __getattr__(name):
+    """``dispatcher`` / ``dispatcher_secondary``: the two module-level GEMM dispatchers of the
+    reference (flextrain/ops/_kernels/_matmul_dispatchers.py:3-4), created on first access instead
+    of at import."""
+    if name in ("dispatcher", "dispatcher_secondary"):
+        if name not in _dispatchers:
+            from ..matmul_dispatcher import CublasLtDispatcher
+            _dispatchers[name] = CublasLtDispatcher(round_multiple=32)
+        return _dispatchers[name]
+    raise AttributeError(f"module {__name__!r} has no attribute {name!r}")
+
+
 __all__ = [
     "build_rope_inv_freq",
+    "destroy_pinned_tensor",
+    "dispatcher",
+    "dispatcher_secondary",
+    "flextrain_embedding_bwd",
+    "flextrain_silu_bwd",
+    "pin_tensor",
     "flextrain_adamw_step",
     "flextrain_copy_expert_counts",
     "flextrain_cross_entropy_loss",

@@ -94,6 +94,20 @@ int fx_glu_fwd(const void* x1, const void* x3, void* out, int64_t n, int in_dt, 
 int fx_glu_bwd(const void* x1, const void* x3, const void* dout, void* dx1, void* dx3, void* act_out,
                int64_t n, int dt, int act, hipStream_t stream);
 
+/* flextrain_silu_bwd (flextrain/ops/_kernels/silu_bwd.py:38-67; kernel :16-35):
+ * din[i] = dout[i] * s * (1 + z[i] * (1 - s)), s = sigmoid(z[i]); n contiguous elements of dtype dt;
+ * din may alias z or dout. */
+int fx_silu_bwd(const void* z, const void* dout, void* din, int64_t n, int dt, hipStream_t stream);
+
+/* flextrain_embedding_bwd (flextrain/ops/_kernels/embed.py:79-122; kernel :5-76).  sorted_tokens: the T
+ * looked-up ids in ascending order; sorted_pos[s]: the row of grad_out (T, D) that sorted position s
+ * came from (both int32, or int64 when indices_are_int64).  grad_weight (V, D) row `token` gets
+ * += scale * (fp32 sum of its grad_out rows).  Strides in elements.  Ids outside [0, V) are skipped. */
+int fx_embedding_bwd(const void* grad_out, const void* sorted_pos, const void* sorted_tokens, int indices_are_int64,
+                     void* grad_weight, int64_t T, int D, int64_t V, int64_t go_row_stride, int64_t go_col_stride,
+                     int64_t gw_row_stride, int64_t gw_col_stride, float scale, int go_dt, int gw_dt,
+                     hipStream_t stream);
+
 /* ---- AdamW ------------------------------------------------------------- */
 
 /* flextrain_adamw_step (flextrain/ops/_kernels/adamw.py:62-102; kernel :5-60).

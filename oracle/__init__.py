@@ -18,7 +18,9 @@ How each function is pinned (tests/test_oracle_*.py, all CPU-only):
                complex multiplication by exp(i*angle) (torch.polar), norm of
                every pair preserved, pos = 0 identity, bwd o fwd = identity.
   glu          torch.nn.functional.silu / gelu(approximate="tanh") and
-               torch.autograd of those (tests/test_gelu_tanh_gated_kernel.py:57-89).
+               torch.autograd of those (tests/test_gelu_tanh_gated_kernel.py:57-89);
+               silu_bwd: torch.autograd of F.silu; embedding_bwd: torch.autograd
+               through F.embedding and a per-token Python loop on a tiny case.
   adamw        torch.optim.AdamW run for several steps
                (flextrain/bench/parity.py:546-577) and the step-1 closed form.
   linear_ce    torch.softmax / argmax, F.cross_entropy (none / sum, ignore_index),

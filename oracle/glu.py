@@ -47,3 +47,19 @@ def gelu_tanh_gated_bwd(x1, x3, dout):
     du = _C * (1.0 + 3.0 * _A * a * a)
     dg = 0.5 * (1.0 + th) + 0.5 * a * (1.0 - th * th) * du
     return (d * b * dg).to(x1.dtype), (d * g).to(x1.dtype), (g * b).to(x1.dtype)
+
+
+def silu_bwd(z, dout):
+    """din = dout * s * (1 + z * (1 - s)), s = sigmoid(z), in fp32, stored in z.dtype
+    (flextrain/ops/_kernels/silu_bwd.py:26-35)."""
+    zf, df = z.float(), dout.float()
+    s = torch.sigmoid(zf)
+    return (df * (s * (1.0 + zf * (1.0 - s)))).to(z.dtype)
+
+
+def embedding_bwd(grad_output, indices, grad_weight, scale=1.0):
+    """grad_weight[token] += scale * (fp32 sum of the grad_output rows of that token), stored in
+    grad_weight.dtype (flextrain/ops/_kernels/embed.py:5-122).  Returns a new tensor."""
+    acc = torch.zeros(grad_weight.shape, dtype=torch.float32)
+    acc.index_add_(0, indices.long(), grad_output.float())
+    return (grad_weight.float() + acc * scale).to(grad_weight.dtype)

@@ -185,6 +185,32 @@ def test_gelu_tanh_gated_matches_library_and_autograd():
     torch.testing.assert_close(act.double(), out.detach(), rtol=1e-5, atol=1e-6)
 
 
+def test_silu_bwd_matches_autograd():
+    g = gen(21)
+    z = randn(g, 64, 33, std=3.0).double().requires_grad_()
+    d = randn(g, 64, 33).double()
+    (gz,) = torch.autograd.grad((F.silu(z) * d).sum(), z)
+    torch.testing.assert_close(o_glu.silu_bwd(z.detach().float(), d.float()).double(), gz, rtol=1e-5, atol=1e-6)
+    assert o_glu.silu_bwd(torch.zeros(4), torch.ones(4)).tolist() == [0.5] * 4      # silu'(0) = 1/2
+
+
+def test_embedding_bwd_matches_autograd_and_loop():
+    g = gen(22)
+    T, D, V = 40, 6, 7
+    go = randn(g, T, D, dtype=torch.float32)
+    idx = torch.randint(0, V, (T,), generator=g)
+    gw0 = randn(g, V, D, dtype=torch.float32)
+    w = torch.zeros(V, D, requires_grad=True)
+    (auto,) = torch.autograd.grad((F.embedding(idx, w) * go).sum(), w)
+    out = o_glu.embedding_bwd(go, idx.int(), gw0, scale=0.25)
+    torch.testing.assert_close(out, gw0 + 0.25 * auto, rtol=1e-6, atol=1e-6)
+    loop = gw0.clone()
+    for t in range(T):
+        loop[idx[t]] += 0.25 * go[t]
+    torch.testing.assert_close(out, loop, rtol=1e-5, atol=1e-6)
+    assert o_glu.embedding_bwd(go, idx, gw0).dtype == gw0.dtype
+
+
 # ------------------------------------------------------------------ AdamW
 def test_adamw_matches_torch_optim_over_steps():
     g = gen(12)
