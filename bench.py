@@ -49,7 +49,7 @@ def _parse():
     ap.add_argument("--no-extra", action="store_true", help="skip the non-headline configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--only", default="", help="comma-separated subset of the non-headline configurations "
-                                               "(c1, c3, c4, c5) to run, e.g. for a profiler pass")
+                                               "(c1, c3, c4, c5, ffn) to run, e.g. for a profiler pass")
     return ap.parse_args()
 
 
@@ -115,6 +115,8 @@ def run_extra(torch, ops, dev, stream, rn, only):
         rows += run_lm_head(torch, dev, stream, rn)
     if want("c5"):
         rows += run_moe(torch, dev, stream, rn)
+    if want("ffn"):
+        rows += run_ffn_dense(torch, dev, stream, rn)
     return rows
 
 
@@ -311,6 +313,40 @@ def run_lm_head(torch, dev, stream, rn):
     del w, g_store, logits, x, x0
     torch.cuda.empty_cache()
     return rows
+
+
+def run_ffn_dense(torch, dev, stream, rn):
+    """Llama-3.1-8B-shaped dense gated FFN block (the GEMMs around the SwiGLU kernels of the headline
+    workload): T = 8192 tokens, d = 4096, F = 14336, bf16 weights and gradients."""
+    import types
+
+    from flextrain_amd.ffn_dense import SwiGLUConfig, SwiGLUFFN
+
+    T, d, F = 8192, 4096, 14336
+    bf = torch.bfloat16
+    h, resid, dy = rn(T, d).to(dev), rn(T, d).to(dev), rn(T, d).to(dev)
+    W = {"w_1": (torch.randn(d, F, device=dev) * 0.02).to(bf), "w_3": (torch.randn(d, F, device=dev) * 0.02).to(bf),
+         "w_2": (torch.randn(F, d, device=dev) * 0.02).to(bf)}
+    G = {"g_" + k[-1]: torch.zeros_like(v) for k, v in W.items()}
+    slot = types.SimpleNamespace(x1=torch.empty(T, F, dtype=bf, device=dev), x3=torch.empty(T, F, dtype=bf, device=dev), aux={})
+    act_buf = torch.empty(T, F, dtype=bf, device=dev)
+    ctx = types.SimpleNamespace(scratch=lambda shape, dtype: act_buf)
+    out = torch.empty(T, d, dtype=bf, device=dev)
+    blk = SwiGLUFFN(SwiGLUConfig(d_model=d, expert_dim=F))
+
+    def fwd():
+        blk.fwd(h, W, resid, out, slot, ctx)
+
+    def bwd():
+        blk.bwd(dy, W, G, slot)
+        blk.bwd_accumulate_w1_w3_grads(h, G, slot)
+
+    unit = 2 * T * d * F
+    ms_f = _time_launches(torch, stream, [fwd], warmup=2, reps=5)
+    ms_b = _time_launches(torch, stream, [bwd], warmup=2, reps=5)
+    return [_op_entry("ffn.dense block fwd (3 GEMMs + SwiGLU, residual in the down-projection epilogue)", 3 * unit, "TFLOP/s", ms_f),
+            _op_entry("ffn.dense block bwd (6 GEMMs + SwiGLU bwd)", 6 * unit, "TFLOP/s", ms_b),
+            _op_entry("ffn.dense block fwd+bwd", 9 * unit, "TFLOP/s", ms_f + ms_b)]
 
 
 def run_moe(torch, dev, stream, rn):

@@ -135,6 +135,9 @@ extern "C" size_t fx_grouped_ws_bytes(int E, int64_t total_rows) {
     return sizeof(int32_t) * (size_t)(2 + E + 2 * (total_rows / 128 + E + 1));
 }
 
+// Row tile: 256 x 256 when experts average 1024 rows or more; otherwise 128 x 128, whose 64 KB of
+// LDS lets two workgroups share a CU, so one's epilogue overlaps the other's K loop (measured
+// 5 % faster over a whole block than 128 x 256 at 512 rows per expert).
 static int rows_bm(int64_t total_rows, int E) { return (total_rows / (E > 0 ? E : 1)) >= 1024 ? 256 : 128; }
 
 extern "C" int fx_grouped_gemm_rows(const void* A, int64_t lda, const void* B, int64_t ldb,
@@ -174,7 +177,7 @@ extern "C" int fx_grouped_gemm_rows(const void* A, int64_t lda, const void* B, i
     }
 #define FX_ROWS_T(TT)                                                                                     \
     if (BM == 256) { if (trans_b) FX_ROWS(TT, 256, 256, 2, 4, false) else FX_ROWS(TT, 256, 256, 2, 4, true) } \
-    else { if (trans_b) FX_ROWS(TT, 128, 256, 2, 2, false) else FX_ROWS(TT, 128, 256, 2, 2, true) }
+    else { if (trans_b) FX_ROWS(TT, 128, 128, 2, 2, false) else FX_ROWS(TT, 128, 128, 2, 2, true) }
     if (dt == DT_BF16) { FX_ROWS_T(bf16) } else { FX_ROWS_T(f16) }
 #undef FX_ROWS_T
 #undef FX_ROWS
