@@ -213,6 +213,75 @@ FX_DEV void mma_step(const T* As, const T* Bs, int row_a0, int row_b0, int lane,
     }
 }
 
+// The same MFMA / LDS-read interleave as mma_step, kept as a running pipeline over all the
+// sub-steps of the K loop: the fragments live in the object, so the MFMAs of the last sub-step of
+// one K-step can run after the workgroup barrier while the first fragments of the next K-step are
+// being read.  Without that, every K-step starts with the matrix pipe idle for the LDS latency of
+// eight waves' first reads.
+template <typename T, int BM, int BN, int WM, int WN, bool A_TR, bool B_TR>
+struct MmaPipe {
+    static constexpr int TM = WM / 32, TN = WN / 32;
+    static constexpr int READS = TM + TN, MFMAS = TM * TN;
+    typedef typename Mfma32<T>::frag frag;
+    typedef short s16x4_t __attribute__((ext_vector_type(4)));
+    typedef short s16x8_t __attribute__((ext_vector_type(8)));
+    typedef __attribute__((address_space(3))) s16x4_t* lds_s16x4_ptr;
+    static_assert(MFMAS >= READS, "a sub-step must have at least as many MFMAs as fragment reads");
+    // one slot of fragments: the operands of one 16-wide sub-step
+    struct Slot {
+        frag a[TM], b[TN];
+    };
+
+    static FX_DEV frag read_k(const T* base, int row0, int ks, int lane) {
+        const int r = row0 + (lane & 31);
+        return *reinterpret_cast<const frag*>(base + r * GEMM_BK + (((ks * 2 + (lane >> 5)) ^ swz(r)) << 3));
+    }
+    static FX_DEV frag read_tr(const T* base, int pitch, int col0, int ks, int lane) {
+        const int grp = lane >> 4, sl = lane & 15;
+        const int n = col0 + 16 * (grp & 1) + 4 * (sl & 3);
+        const int k = 16 * ks + 8 * (grp >> 1) + (sl >> 2);
+        const int off = (((n >> 3) ^ (swz_tr(k) % (pitch / 8))) << 3) + (n & 7);
+        const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(base + k * pitch + off));
+        const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(base + (k + 4) * pitch + off));
+        const s16x8_t both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        return __builtin_bit_cast(frag, both);
+    }
+    // Read R of a sub-step, in the order the MFMAs first use the fragments (A-fragment-major
+    // MFMA order): a[0], b[0] .. b[TN-1], a[1] .. a[TM-1].
+    template <int R>
+    static FX_DEV void fetch_one(Slot& f, const T* As, const T* Bs, int ks, int row_a0, int row_b0, int lane) {
+        constexpr bool IS_A = R == 0 || R > TN;
+        constexpr int IDX = R == 0 ? 0 : (R <= TN ? R - 1 : R - TN);
+        if constexpr (IS_A) f.a[IDX] = A_TR ? read_tr(As, BM, row_a0 + IDX * 32, ks, lane) : read_k(As, row_a0 + IDX * 32, ks, lane);
+        else f.b[IDX] = B_TR ? read_tr(Bs, BN, row_b0 + IDX * 32, ks, lane) : read_k(Bs, row_b0 + IDX * 32, ks, lane);
+    }
+    template <int R = 0>
+    static FX_DEV void fetch_all(Slot& f, const T* As, const T* Bs, int ks, int row_a0, int row_b0, int lane) {
+        if constexpr (R < READS) {
+            fetch_one<R>(f, As, Bs, ks, row_a0, row_b0, lane);
+            fetch_all<R + 1>(f, As, Bs, ks, row_a0, row_b0, lane);
+        }
+    }
+    // MFMAs of the sub-step whose fragments sit in `cur`; with FETCH, the fragments of sub-step
+    // ks_f of tiles (As_f, Bs_f) are read into `nxt`, one read after each of the first MFMAs.
+    template <bool FETCH, int M = 0>
+    static FX_DEV void sub(f32x16_t (&acc)[TM][TN], const Slot& cur, Slot& nxt, const T* As_f, const T* Bs_f, int ks_f,
+                           int row_a0, int row_b0, int lane) {
+        if constexpr (M < MFMAS) {
+            constexpr int i = M / TN, j = M % TN;
+            __builtin_amdgcn_sched_barrier(0);
+            acc[i][j] = Mfma32<T>::run(cur.b[j], cur.a[i], acc[i][j]);   // transposed tile: rows = n, columns = m
+            if constexpr (FETCH && M < READS) {
+                __builtin_amdgcn_sched_barrier(0);
+                fetch_one<M>(nxt, As_f, Bs_f, ks_f, row_a0, row_b0, lane);
+            }
+            sub<FETCH, M + 1>(acc, cur, nxt, As_f, Bs_f, ks_f, row_a0, row_b0, lane);
+        } else {
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+};
+
 // Epilogue.  The accumulators hold the transposed tile (MFMA is called with the B fragment
 // first): lane l, register v of acc[i][j] is D[row0 + 32i + l%32][col0 + 32j + 8*(v/4) + 4*(l/32) + v%4],
 // i.e. a lane owns groups of 4 consecutive columns.  Each wave stages one 32-row band at a time in
@@ -312,14 +381,39 @@ FX_DEV void gemm_tile2(const OperandView<T>& A, const OperandView<T>& B, const T
         if (!B_MN) tile_load_direct<T, BN, NW>(B, kt * GEMM_BK, buf + BM * GEMM_BK, wave, lane);
         else tile_load_direct_tr<T, BN, NW>(B, kt * GEMM_BK, buf + BM * GEMM_BK, wave, lane);
     };
-    if (nfull > 0) issue(0, smem);
-    for (int kt = 0; kt < nfull; ++kt) {
-        T* cur = smem + (kt & 1) * BUF;
-        T* nxt = smem + ((kt + 1) & 1) * BUF;
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's loads of step kt have landed
-        __syncthreads();                                  // everyone's have, and buffer `nxt` is no longer read
-        if (kt + 1 < nfull) issue(kt + 1, nxt);
-        mma_step<T, BM, BN, WM, WN, A_MN, B_MN>(cur, cur + BM * GEMM_BK, wm * WM, wn * WN, lane, acc);
+    static_assert(GEMM_BK == 64, "the pipeline below is written out for four sub-steps per K-step");
+    if (nfull > 0) {
+        typedef MmaPipe<T, BM, BN, WM, WN, A_MN, B_MN> Pipe;
+        typename Pipe::Slot f0, f1;
+        const int ra = wm * WM, rb = wn * WN;
+        issue(0, smem);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (nfull > 1) issue(1, smem + BUF);
+        Pipe::fetch_all(f0, smem, smem + BM * GEMM_BK, 0, ra, rb, lane);
+        for (int kt = 0; kt + 1 < nfull; ++kt) {
+            T* cur = smem + (kt & 1) * BUF;
+            T* nxt = smem + ((kt + 1) & 1) * BUF;
+            T* curb = cur + BM * GEMM_BK;
+            Pipe::template sub<true>(acc, f0, f1, cur, curb, 1, ra, rb, lane);
+            Pipe::template sub<true>(acc, f1, f0, cur, curb, 2, ra, rb, lane);
+            Pipe::template sub<true>(acc, f0, f1, cur, curb, 3, ra, rb, lane);
+            // Every read of `cur` has been issued.  Once they and this wave's loads of step kt+1 have
+            // landed, the barrier makes `nxt` readable and `cur` writable for everyone; the MFMAs of
+            // the last sub-step then run while the first fragments of step kt+1 are read.
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+            __syncthreads();
+            if (kt + 2 < nfull) issue(kt + 2, cur);
+            Pipe::template sub<true>(acc, f1, f0, nxt, nxt + BM * GEMM_BK, 0, ra, rb, lane);
+        }
+        {   // last full K-step: nothing follows it in these buffers
+            T* cur = smem + ((nfull - 1) & 1) * BUF;
+            T* curb = cur + BM * GEMM_BK;
+            Pipe::template sub<true>(acc, f0, f1, cur, curb, 1, ra, rb, lane);
+            Pipe::template sub<true>(acc, f1, f0, cur, curb, 2, ra, rb, lane);
+            Pipe::template sub<true>(acc, f0, f1, cur, curb, 3, ra, rb, lane);
+            Pipe::template sub<false>(acc, f1, f0, cur, curb, 0, ra, rb, lane);
+        }
     }
     if (nfull * GEMM_BK < K) {  // K tail: through registers into the K-contiguous layout, zero-filled past K
         Staged2<BM, NT> sa;
