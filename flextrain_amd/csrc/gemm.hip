@@ -17,28 +17,6 @@
 
 namespace fx {
 
-// blockIdx.x -> (tile_m, tile_n).  Workgroups are dealt round-robin to the 8 XCDs,
-// each with its own L2: give every XCD a contiguous band of tile indices and walk
-// the band in groups of GROUP_M tile-rows so concurrently resident workgroups
-// share A rows and B columns in L2.
-FX_DEV void tile_coords(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
-    const int total = tiles_m * tiles_n;
-    constexpr int XCDS = 8;
-    int p = pid;
-    if (total >= XCDS * 4) {
-        const int per = total / XCDS;          // band length; the remainder keeps its order
-        const int body = per * XCDS;
-        if (pid < body) p = (pid % XCDS) * per + pid / XCDS;
-    }
-    constexpr int GROUP_M = 8;
-    const int width = GROUP_M * tiles_n;
-    const int group = p / width;
-    const int first_m = group * GROUP_M;
-    const int gsz = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
-    tm = first_m + (p % width) % gsz;
-    tn = (p % width) / gsz;
-}
-
 // blockIdx.y selects a K split: split s covers k in [s*k_per_split, min(K, (s+1)*k_per_split)) and,
 // when there is more than one, writes its fp32 partial product to PART + s*M*N (row stride N).
 template <typename T, typename TD, int BM, int BN, int WAVES_M, int WAVES_N, bool A_MN, bool B_MN>

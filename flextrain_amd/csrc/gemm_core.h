@@ -54,6 +54,10 @@ struct OperandView {
     int64_t ld;
     int ext;
     int origin;
+    // Two-matrix tile (loaders instantiated with DUAL): tile rows >= half come from the matrix
+    // that starts half_delta elements after `base`, at index origin + row - half.
+    int half = 0;
+    int64_t half_delta = 0;
 };
 
 // Registers that park one K-step of one operand tile (ROWS x 64 elements):

@@ -41,7 +41,7 @@ FX_DEV void load_to_lds16(const void* gptr, void* lds_base) {
 
 // Direct copy of a ROWS x 64 K-contiguous tile.  One wave instruction covers 8 rows
 // (8 lanes per row); instruction j of wave w covers rows (j*NW + w)*8 ...
-template <typename T, int ROWS, int NW>
+template <typename T, int ROWS, int NW, bool DUAL = false>
 FX_DEV void tile_load_direct(const OperandView<T>& op, int k0, T* lds, int wave, int lane) {
     constexpr int NI = ROWS / 8 / NW;
     static_assert(ROWS % (8 * NW) == 0, "tile rows must split evenly over the waves");
@@ -49,10 +49,13 @@ FX_DEV void tile_load_direct(const OperandView<T>& op, int k0, T* lds, int wave,
 #pragma unroll
     for (int j = 0; j < NI; ++j) {
         const int r = (j * NW + wave) * 8 + rr;
-        int g = op.origin + r;
+        const bool second = DUAL && r >= op.half;
+        int g = op.origin + (second ? r - op.half : r);
         g = g < op.ext ? g : op.ext - 1;
         const int c = pos ^ swz(r);
-        load_to_lds16(op.base + (int64_t)g * op.ld + k0 + c * 8, lds + (j * NW + wave) * 8 * GEMM_BK);
+        const T* src = op.base + (int64_t)g * op.ld + k0 + c * 8;
+        if (second) src += op.half_delta;
+        load_to_lds16(src, lds + (j * NW + wave) * 8 * GEMM_BK);
     }
 }
 
@@ -60,7 +63,7 @@ FX_DEV void tile_load_direct(const OperandView<T>& op, int k0, T* lds, int wave,
 // chunk c at position c ^ ((k & 3) << 2).  One wave instruction covers 1024 / (2*ROWS) k-rows.
 FX_DEV int swz_tr(int k) { return (k & 3) << 2; }
 
-template <typename T, int ROWS, int NW>
+template <typename T, int ROWS, int NW, bool DUAL = false>
 FX_DEV void tile_load_direct_tr(const OperandView<T>& op, int k0, T* lds, int wave, int lane) {
     constexpr int NI = ROWS / 8 / NW;           // instructions per wave: ROWS * 128 bytes in all
     constexpr int CPR = ROWS / 8;               // 16-byte chunks per LDS row
@@ -72,9 +75,12 @@ FX_DEV void tile_load_direct_tr(const OperandView<T>& op, int k0, T* lds, int wa
         const int q = j * NW + wave;
         const int k = q * KPI + kin;
         const int c = pos ^ (swz_tr(k) % CPR);
-        int g = op.origin + c * 8;
+        const bool second = DUAL && c * 8 >= op.half;
+        int g = op.origin + (second ? c * 8 - op.half : c * 8);
         g = g + 8 <= op.ext ? g : op.ext - 8;
-        load_to_lds16(op.base + (int64_t)(k0 + k) * op.ld + g, lds + q * 512);
+        const T* src = op.base + (int64_t)(k0 + k) * op.ld + g;
+        if (second) src += op.half_delta;
+        load_to_lds16(src, lds + q * 512);
     }
 }
 
@@ -354,9 +360,12 @@ constexpr size_t gemm2_lds_bytes() {
     return tiles > epi ? tiles : epi;
 }
 
-template <typename T, typename TD, int BM, int BN, int WAVES_M, int WAVES_N, bool A_MN, bool B_MN>
-FX_DEV void gemm_tile2(const OperandView<T>& A, const OperandView<T>& B, const TD* C, TD* D, int64_t ldc,
-                       int64_t ldd, int M, int N, int K, float alpha, float beta, T* smem) {
+// K loop of one workgroup tile: leaves the fp32 accumulators of this wave's sub-tile in `acc`
+// (transposed MFMA layout, see epilogue_tile).  B_DUAL: the B tile's second half comes from a
+// second matrix (OperandView::half); K must then be a multiple of 64.
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_MN, bool B_MN, bool B_DUAL = false>
+FX_DEV void gemm_mainloop2(const OperandView<T>& A, const OperandView<T>& B, int K, T* smem,
+                           f32x16_t (&acc)[BM / WAVES_M / 32][BN / WAVES_N / 32]) {
     constexpr int NW = WAVES_M * WAVES_N, NT = NW * 64;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     constexpr int TM = WM / 32, TN = WN / 32;
@@ -366,7 +375,6 @@ FX_DEV void gemm_tile2(const OperandView<T>& A, const OperandView<T>& B, const T
     const int wave = tid >> 6;
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
 
-    f32x16_t acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -378,8 +386,8 @@ FX_DEV void gemm_tile2(const OperandView<T>& A, const OperandView<T>& B, const T
     auto issue = [&](int kt, T* buf) {
         if (!A_MN) tile_load_direct<T, BM, NW>(A, kt * GEMM_BK, buf, wave, lane);
         else tile_load_direct_tr<T, BM, NW>(A, kt * GEMM_BK, buf, wave, lane);
-        if (!B_MN) tile_load_direct<T, BN, NW>(B, kt * GEMM_BK, buf + BM * GEMM_BK, wave, lane);
-        else tile_load_direct_tr<T, BN, NW>(B, kt * GEMM_BK, buf + BM * GEMM_BK, wave, lane);
+        if (!B_MN) tile_load_direct<T, BN, NW, B_DUAL>(B, kt * GEMM_BK, buf + BM * GEMM_BK, wave, lane);
+        else tile_load_direct_tr<T, BN, NW, B_DUAL>(B, kt * GEMM_BK, buf + BM * GEMM_BK, wave, lane);
     };
     static_assert(GEMM_BK == 64, "the pipeline below is written out for four sub-steps per K-step");
     if (nfull > 0) {
@@ -415,7 +423,7 @@ FX_DEV void gemm_tile2(const OperandView<T>& A, const OperandView<T>& B, const T
             Pipe::template sub<false>(acc, f1, f0, cur, curb, 0, ra, rb, lane);
         }
     }
-    if (nfull * GEMM_BK < K) {  // K tail: through registers into the K-contiguous layout, zero-filled past K
+    if (!B_DUAL && nfull * GEMM_BK < K) {  // K tail: through registers into the K-contiguous layout, zero-filled past K
         Staged2<BM, NT> sa;
         Staged2<BN, NT> sb;
         T* buf = smem + (nfull & 1) * BUF;
@@ -428,7 +436,114 @@ FX_DEV void gemm_tile2(const OperandView<T>& A, const OperandView<T>& B, const T
     }
     __syncthreads();  // every wave is past its last LDS read: the buffers become epilogue staging
     static_assert(gemm2_lds_bytes<T, BM, BN, WAVES_M, WAVES_N>() <= 160 * 1024, "tile configuration exceeds the 160 KB of LDS");
+}
+
+template <typename T, typename TD, int BM, int BN, int WAVES_M, int WAVES_N, bool A_MN, bool B_MN>
+FX_DEV void gemm_tile2(const OperandView<T>& A, const OperandView<T>& B, const TD* C, TD* D, int64_t ldc,
+                       int64_t ldd, int M, int N, int K, float alpha, float beta, T* smem) {
+    constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    f32x16_t acc[WM / 32][WN / 32];
+    gemm_mainloop2<T, BM, BN, WAVES_M, WAVES_N, A_MN, B_MN>(A, B, K, smem, acc);
     epilogue_tile<T, TD, WM, WN>(acc, C, D, ldc, ldd, A.origin + wm * WM, B.origin + wn * WN, M, N, alpha, beta, smem, wave, lane);
+}
+
+// Two GEMMs that share A, fused with the gated activation:
+//   P1 = A * op(B1),  P2 = A * op(B2)  (both stored, rounded to T),  ACT = act(gate) * value
+// with (gate, value) = (P1, P2) when gate_first, else (P2, P1), evaluated from the ROUNDED P1 / P2
+// exactly as a separate activation kernel reading them back would.  The workgroup's BN columns are
+// BN/2 columns of B1 followed by the same BN/2 columns of B2 (OperandView::half of `B`): waves
+// with wn < WAVES_N/2 accumulate P1, the others P2, and wave w pairs with wave w ^ (WAVES_N/2).
+// Per 32-row band every wave stages its fp32 results in LDS; after a barrier each wave of a pair
+// finishes 16 of the band's rows: reads both stagings, rounds, applies the activation and stores
+// the three outputs as 16-byte accesses.  Needs K % 64 == 0, Nh % 8 == 0, 16-byte aligned rows.
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool B_MN, int ACT>
+FX_DEV void gemm_tile2_glu(const OperandView<T>& A, const OperandView<T>& B, T* P1, T* P2, int64_t ldp, T* ACTO,
+                           int64_t ldact, int M, int Nh, int K, bool gate_first, T* smem) {
+    constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+    constexpr int TM = WM / 32, TN = WN / 32;
+    constexpr int HW = WAVES_N / 2;                 // waves per half along n
+    constexpr int PITCH = WN + 4, GROUPS = WN / 8;
+    constexpr int PER_LANE = 16 * GROUPS / 64;
+    static_assert(WAVES_N % 2 == 0 && (16 * GROUPS) % 64 == 0, "unsupported wave layout for the gated epilogue");
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    f32x16_t acc[TM][TN];
+    gemm_mainloop2<T, BM, BN, WAVES_M, WAVES_N, false, B_MN, true>(A, B, K, smem, acc);
+
+    float* stage = reinterpret_cast<float*>(smem) + wave * 32 * PITCH;
+    const bool second = wn >= HW;
+    const float* s1 = reinterpret_cast<float*>(smem) + (second ? wave - HW : wave) * 32 * PITCH;
+    const float* s2 = s1 + HW * 32 * PITCH;
+    const int row_base = A.origin + wm * WM, col_base = B.origin + (wn % HW) * WN;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const f32x4_t q = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+                *reinterpret_cast<f32x4_t*>(stage + (lane & 31) * PITCH + j * 32 + 8 * g + 4 * (lane >> 5)) = q;
+            }
+        __syncthreads();
+#pragma unroll
+        for (int t = 0; t < PER_LANE; ++t) {
+            const int id = t * 64 + lane;
+            const int rr = (second ? 16 : 0) + id / GROUPS, cg = id % GROUPS;
+            const int row = row_base + i * 32 + rr, col = col_base + cg * 8;
+            if (row < M && col < Nh) {
+                const f32x4_t a0 = *reinterpret_cast<const f32x4_t*>(s1 + rr * PITCH + cg * 8);
+                const f32x4_t a1 = *reinterpret_cast<const f32x4_t*>(s1 + rr * PITCH + cg * 8 + 4);
+                const f32x4_t b0 = *reinterpret_cast<const f32x4_t*>(s2 + rr * PITCH + cg * 8);
+                const f32x4_t b1 = *reinterpret_cast<const f32x4_t*>(s2 + rr * PITCH + cg * 8 + 4);
+                float v1[8], v2[8], y[8];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    v1[e] = round_to<T>(a0[e]); v1[4 + e] = round_to<T>(a1[e]);
+                    v2[e] = round_to<T>(b0[e]); v2[4 + e] = round_to<T>(b1[e]);
+                }
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    y[e] = gate_first ? glu_fwd_elem<T, ACT>(v1[e], v2[e]) : glu_fwd_elem<T, ACT>(v2[e], v1[e]);
+                store_f32<T, 8>(P1 + (int64_t)row * ldp + col, v1);
+                store_f32<T, 8>(P2 + (int64_t)row * ldp + col, v2);
+                store_f32<T, 8>(ACTO + (int64_t)row * ldact + col, y);
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// ---------------------------------------------------------------- workgroup -> tile maps
+// blockIdx.x -> (tile_m, tile_n).  Workgroups are dealt round-robin to the 8 XCDs,
+// each with its own L2: give every XCD a contiguous band of tile indices and walk
+// the band in groups of GROUP_M tile-rows so concurrently resident workgroups
+// share A rows and B columns in L2.
+FX_DEV void tile_coords(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
+    const int total = tiles_m * tiles_n;
+    constexpr int XCDS = 8;
+    int p = pid;
+    if (total >= XCDS * 4) {
+        const int per = total / XCDS;          // band length; the remainder keeps its order
+        const int body = per * XCDS;
+        if (pid < body) p = (pid % XCDS) * per + pid / XCDS;
+    }
+    constexpr int GROUP_M = 8;
+    const int width = GROUP_M * tiles_n;
+    const int group = p / width;
+    const int first_m = group * GROUP_M;
+    const int gsz = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
+    tm = first_m + (p % width) % gsz;
+    tn = (p % width) / gsz;
+}
+
+// pid -> position in the logical order: XCD x (= pid % 8) walks positions [x*per, (x+1)*per).
+FX_DEV int xcd_band(int pid, int total) {
+    constexpr int XCDS = 8;
+    if (total < XCDS * 4) return pid;
+    const int per = total / XCDS, body = per * XCDS;
+    return pid < body ? (pid % XCDS) * per + pid / XCDS : pid;
 }
 
 }  // namespace fx

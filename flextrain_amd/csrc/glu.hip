@@ -9,27 +9,6 @@
 
 namespace fx {
 
-enum : int { ACT_SILU = 0, ACT_GELU_TANH = 1 };
-
-FX_DEV float fast_sigmoid(float x) {
-    // 1 / (1 + 2^(-x*log2 e)); v_exp_f32 + v_rcp_f32, ~1 ulp each.
-    return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x));
-}
-
-template <typename T, int ACT>
-FX_DEV float glu_fwd_elem(float x1, float x3) {
-    if (ACT == ACT_SILU) {
-        const float s = fast_sigmoid(x1);
-        return (x1 * s) * x3;
-    } else {
-        const float cu = x1 * x1 * x1;
-        const float u = 0.7978845608028654f * (x1 + 0.044715f * cu);
-        const float th = 2.0f * fast_sigmoid(2.0f * u) - 1.0f;
-        const float g = 0.5f * x1 * (1.0f + th);
-        return g * x3;
-    }
-}
-
 template <typename T, int ACT>
 FX_DEV void glu_bwd_elem(float x1, float x3, float dout, float& dx1, float& dx3, float& act) {
     if (ACT == ACT_SILU) {

@@ -68,14 +68,6 @@ __global__ __launch_bounds__(256) void grouped_plan_kernel(const int32_t* __rest
     if (threadIdx.x == 0) { OFFSETS[E] = carry_r; NTILES[0] = carry_t; }
 }
 
-// pid -> position in the logical order: XCD x (= pid % 8) walks positions [x*per, (x+1)*per).
-FX_DEV int xcd_band(int pid, int total) {
-    constexpr int XCDS = 8;
-    if (total < XCDS * 4) return pid;
-    const int per = total / XCDS, body = per * XCDS;
-    return pid < body ? (pid % XCDS) * per + pid / XCDS : pid;
-}
-
 template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool B_MN>
 __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void grouped_rows_kernel(
     const T* __restrict__ A, int64_t lda, const T* __restrict__ B, int64_t ldb, int64_t b_expert_stride,
@@ -101,6 +93,33 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void grouped_rows_kernel(
     OperandView<T> b{B + (int64_t)e * b_expert_stride, ldb, N, tn * BN};
     const T* c = C ? C + row0 * ldc : nullptr;
     gemm_tile2<T, T, BM, BN, WAVES_M, WAVES_N, false, B_MN>(a, b, c, D + row0 * ldd, ldc, ldd, rows, N, K, alpha, beta, smem);
+}
+
+// Up projection of every expert with the SwiGLU in the epilogue: the expert's weight holds two
+// Nh-row (or Nh-column) halves b2_delta elements apart; P1 / P2 receive the two pre-activation
+// halves and ACTO the gated product (see gemm_tile2_glu).
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool B_MN>
+__global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void grouped_rows_glu_kernel(
+    const T* __restrict__ A, int64_t lda, const T* __restrict__ B, int64_t ldb, int64_t b_expert_stride,
+    int64_t b2_delta, T* P1, T* P2, int64_t ldp, T* ACTO, int64_t ldact, const int32_t* __restrict__ NTILES,
+    const int32_t* __restrict__ OFFSETS, const int32_t* __restrict__ TILES, int Nh, int K, int gate_first,
+    int tiles_n) {
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T* smem = reinterpret_cast<T*>(smem_raw);
+    const int total = NTILES[0] * tiles_n;
+    const int pid = blockIdx.x;
+    if (pid >= total) return;
+    const int p = xcd_band(pid, total);
+    const int tile = p / tiles_n, tn = p % tiles_n;
+    const int e = TILES[2 * tile];
+    const int m0 = TILES[2 * tile + 1];
+    const int64_t row0 = OFFSETS[e];
+    const int rows = OFFSETS[e + 1] - OFFSETS[e];
+    OperandView<T> a{A + row0 * lda, lda, rows, m0};
+    OperandView<T> b{B + (int64_t)e * b_expert_stride, ldb, Nh, tn * (BN / 2), BN / 2, b2_delta};
+    gemm_tile2_glu<T, BM, BN, WAVES_M, WAVES_N, B_MN, ACT_SILU>(a, b, P1 + row0 * ldp, P2 + row0 * ldp, ldp,
+                                                                ACTO + row0 * ldact, ldact, rows, Nh, K,
+                                                                gate_first != 0, smem);
 }
 
 template <typename T, typename TG, int BM, int BN, int WAVES_M, int WAVES_N>
@@ -182,6 +201,49 @@ extern "C" int fx_grouped_gemm_rows(const void* A, int64_t lda, const void* B, i
 #undef FX_ROWS_T
 #undef FX_ROWS
     FX_CHECK_LAUNCH("fx_grouped_gemm_rows");
+    return 0;
+}
+
+extern "C" int fx_grouped_gemm_rows_glu(const void* A, int64_t lda, const void* B, int64_t ldb, int64_t b_expert_stride,
+                                        int trans_b, int64_t b2_delta, void* P1, void* P2, int64_t ldp, void* act,
+                                        int64_t ldact, const int32_t* counts, int E, int64_t total_rows, int Nh, int K,
+                                        int gate_first, int dt, void* ws, size_t ws_bytes, hipStream_t stream) {
+    if (E <= 0 || total_rows < 0 || Nh <= 0 || K <= 0) FX_FAIL("fx_grouped_gemm_rows_glu: bad shape");
+    if (total_rows == 0) return 0;
+    if (!A || !B || !P1 || !P2 || !act || !counts) FX_FAIL("fx_grouped_gemm_rows_glu: null pointer");
+    if (!ws || ws_bytes < fx_grouped_ws_bytes(E, total_rows)) FX_FAIL("fx_grouped_gemm_rows_glu: workspace too small");
+    if (dt != DT_BF16 && dt != DT_F16) FX_FAIL("fx_grouped_gemm_rows_glu: bf16 or fp16 only");
+    if (!aligned16(A) || !aligned16(B) || !aligned16(P1) || !aligned16(P2) || !aligned16(act) || (lda & 7) || (ldb & 7) ||
+        (ldp & 7) || (ldact & 7) || (K & 63) || (Nh & 7) || (b_expert_stride & 7) || (b2_delta & 7))
+        FX_FAIL("fx_grouped_gemm_rows_glu: needs K %% 64 == 0, N %% 8 == 0, strides %% 8 == 0 and 16-byte aligned operands");
+    GroupedWs w = split_ws(ws, E);
+    const int BM = rows_bm(total_rows, E);
+    grouped_plan_kernel<<<1, 256, 0, stream>>>(counts, E, BM, w.ntiles, w.offsets, w.tiles);
+    FX_CHECK_LAUNCH("fx_grouped_gemm_rows_glu(plan)");
+    const unsigned max_tiles = (unsigned)(total_rows / BM + E);
+#define FX_GLU(TT, BM_, BN_, WM_, WN_, BMN)                                                               \
+    {                                                                                                     \
+        auto kern = grouped_rows_glu_kernel<TT, BM_, BN_, WM_, WN_, BMN>;                                 \
+        constexpr size_t lds = gemm2_lds_bytes<TT, BM_, BN_, WM_, WN_>();                                 \
+        static bool attr_set = false;                                                                     \
+        if (!attr_set) {                                                                                  \
+            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                \
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);              \
+            attr_set = true;                                                                              \
+        }                                                                                                 \
+        const int tiles_n = cdiv_i(Nh, BN_ / 2);                                                          \
+        kern<<<dim3(max_tiles * (unsigned)tiles_n), WM_ * WN_ * 64, lds, stream>>>(                       \
+            reinterpret_cast<const TT*>(A), lda, reinterpret_cast<const TT*>(B), ldb, b_expert_stride,    \
+            b2_delta, reinterpret_cast<TT*>(P1), reinterpret_cast<TT*>(P2), ldp, reinterpret_cast<TT*>(act), \
+            ldact, w.ntiles, w.offsets, w.tiles, Nh, K, gate_first, tiles_n);                             \
+    }
+#define FX_GLU_T(TT)                                                                                      \
+    if (BM == 256) { if (trans_b) FX_GLU(TT, 256, 256, 2, 4, false) else FX_GLU(TT, 256, 256, 2, 4, true) } \
+    else { if (trans_b) FX_GLU(TT, 128, 128, 2, 2, false) else FX_GLU(TT, 128, 128, 2, 2, true) }
+    if (dt == DT_BF16) { FX_GLU_T(bf16) } else { FX_GLU_T(f16) }
+#undef FX_GLU_T
+#undef FX_GLU
+    FX_CHECK_LAUNCH("fx_grouped_gemm_rows_glu");
     return 0;
 }
 

@@ -4,7 +4,8 @@ Host-side mirror of the reference block (flextrain/nn/blocks/ffn_dense.py:57-301
 method names, argument meaning, saved activations (``slot.x1`` / ``slot.x3``), the
 ``skip_grads`` / ``capture_xy`` contract and the hand-off of ``dx1_up`` / ``dx3_up`` through
 ``slot.aux``.  Every GEMM goes through the MFMA dispatcher (`dispatch_matmul`), with the residual
-add folded into the down projection (``beta = 1`` on the residual operand) and the weight
+add folded into the down projection (``beta = 1`` on the residual operand), the gate and up projections run as one launch with the
+activation in its epilogue when the shapes allow (``fuse_gate_up``), and the weight
 gradients accumulated in place (``beta = 1`` on the gradient itself); the gated activation and
 its backward are the SwiGLU / GELU-tanh kernels of :mod:`flextrain_amd.ops`.
 
@@ -19,6 +20,7 @@ from typing import Mapping, MutableMapping, Sequence
 import torch
 
 from . import ops
+from .ops.grouped import dual_glu_supported, flextrain_gemm_dual_glu
 
 
 @dataclass(frozen=True)
@@ -44,11 +46,12 @@ def _stream_ptr(t):
 class SwiGLUFFN:
     """Gate / up / down projections around the gated activation."""
 
-    def __init__(self, cfg: SwiGLUConfig, dispatcher=None):
+    def __init__(self, cfg: SwiGLUConfig, dispatcher=None, fuse_gate_up: bool = True):
         if cfg.activation not in ("silu", "gelu_tanh"):
             raise ValueError(f"SwiGLUFFN: unsupported activation {cfg.activation!r}")
         self.cfg = cfg
         self._dispatcher = dispatcher
+        self.fuse_gate_up = fuse_gate_up
 
     @property
     def dispatcher(self):
@@ -72,10 +75,16 @@ class SwiGLUFFN:
             ctx=None):
         """Writes ``slot.x1``, ``slot.x3`` and returns ``out_tensor`` (which may be the residual
         tensor itself: the down projection reads each residual element before writing it)."""
-        self._mm(ffn_norm_output, weights["w_1"], slot.x1)
-        self._mm(ffn_norm_output, weights["w_3"], slot.x3)
         scratch = ctx.scratch(slot.x1.shape, slot.x1.dtype) if ctx is not None else torch.empty_like(slot.x1)
-        act = self._act_fwd(slot.x1, slot.x3, scratch)
+        w1, w3 = weights["w_1"], weights["w_3"]
+        if self.fuse_gate_up and dual_glu_supported(ffn_norm_output, w1, w3, slot.x1, slot.x3, scratch):
+            # one launch: both projections and the activation from their rounded results
+            act = flextrain_gemm_dual_glu(ffn_norm_output, w1, w3, slot.x1, slot.x3, scratch,
+                                          activation=self.cfg.activation, gate_first=True)
+        else:
+            self._mm(ffn_norm_output, w1, slot.x1)
+            self._mm(ffn_norm_output, w3, slot.x3)
+            act = self._act_fwd(slot.x1, slot.x3, scratch)
         return self._mm(act, weights["w_2"], out_tensor, C=attn_output_with_residual, beta=1.0)
 
     def fwd_recompute_x1x3(self, ffn_norm_output, weights, slot, *, recompute_x1: bool, recompute_x3: bool) -> None:

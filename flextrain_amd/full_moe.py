@@ -15,7 +15,12 @@ from typing import Any, Callable, Mapping, MutableMapping
 import torch
 
 from .matmul_dispatcher import CublasLtDispatcher
-from .ops.grouped import flextrain_grouped_gemm_rows, flextrain_grouped_gemm_wgrad
+from .ops.grouped import (
+    flextrain_grouped_gemm_rows,
+    flextrain_grouped_gemm_rows_glu,
+    flextrain_grouped_gemm_wgrad,
+    grouped_glu_supported,
+)
 from .ops.moe import (
     flextrain_fused_topk_softmax,
     flextrain_load_balance_bwd,
@@ -99,12 +104,15 @@ def swiglu_expert_loop_fwd(scattered_x, x_preact_buf, w_up, w_down, expert_count
     counts = _device_counts(expert_counts_cpu, expert_counts_gpu)
     with torch.cuda.stream(primary_stream):
         pre = x_preact_buf[:TK]
-        flextrain_grouped_gemm_rows(scattered_x, w_up.transpose(1, 2), counts, pre)
         if x_act_even is not None and x_act_even.shape[0] >= TK and x_act_even.shape[1] == F:
             act = x_act_even[:TK]
         else:
             act = torch.empty((TK, F), dtype=scattered_x.dtype, device=scattered_x.device)
-        flextrain_swiglu_moe_fwd(pre, out=act)
+        if grouped_glu_supported(scattered_x, w_up, pre, act):
+            flextrain_grouped_gemm_rows_glu(scattered_x, w_up, counts, pre, act)   # SwiGLU in the GEMM epilogue
+        else:
+            flextrain_grouped_gemm_rows(scattered_x, w_up.transpose(1, 2), counts, pre)
+            flextrain_swiglu_moe_fwd(pre, out=act)
         flextrain_grouped_gemm_rows(act, w_down.transpose(1, 2), counts, scattered_x)
 
 

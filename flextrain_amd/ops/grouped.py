@@ -79,3 +79,80 @@ def flextrain_grouped_gemm_wgrad(A, B, G, counts, alpha=1.0, beta=1.0):
                                      dtype_enum(A.dtype), ptr(ws), nbytes, stream_ptr(A.device))
     check(rc, "fx_grouped_gemm_wgrad")
     return G
+
+
+
+def _b_layout(B):
+    if B.stride(-1) == 1:
+        return 0, B.stride(-2)
+    if B.stride(-2) == 1:
+        return 1, B.stride(-1)
+    raise ValueError("the weight must be row-major or column-major")
+
+
+def grouped_glu_supported(A, w_up, pre, act):
+    """Whether :func:`flextrain_grouped_gemm_rows_glu` can take these tensors (else the caller
+    runs the GEMM and the activation kernel separately)."""
+    F = act.shape[1]
+    K = A.shape[1]
+    return (A.dtype in (torch.bfloat16, torch.float16) and A.dtype == w_up.dtype == pre.dtype == act.dtype
+            and K % 64 == 0 and F % 8 == 0 and A.stride(1) == 1 and pre.stride(1) == 1 and act.stride(1) == 1
+            and A.stride(0) % 8 == 0 and pre.stride(0) % 8 == 0 and act.stride(0) % 8 == 0
+            and w_up.is_contiguous() and all(t.data_ptr() % 16 == 0 for t in (A, w_up, pre, act)))
+
+
+def flextrain_grouped_gemm_rows_glu(A, w_up, counts, pre, act):
+    """Expert up-projection and SwiGLU in one launch: ``pre[rows_e] = A[rows_e] @ w_up[e].T``
+    (packed ``[value (F) | gate (F)]`` like ``w_up (E, 2F, K)``) and ``act = silu(gate) * value``,
+    the activation evaluated from the rounded ``pre`` as the separate kernel would."""
+    _rowmajor(A, "A"), _rowmajor(pre, "pre"), _rowmajor(act, "act")
+    if w_up.dim() != 3 or not w_up.is_contiguous():
+        raise ValueError("w_up must be a contiguous (E, 2F, K) tensor")
+    E, F2, K = w_up.shape
+    F = F2 // 2
+    TK = A.shape[0]
+    if A.shape[1] != K or tuple(pre.shape) != (TK, F2) or tuple(act.shape) != (TK, F):
+        raise ValueError(f"shape mismatch: A {tuple(A.shape)}, w_up {tuple(w_up.shape)}, pre {tuple(pre.shape)}, "
+                         f"act {tuple(act.shape)}")
+    ws, nbytes = _workspace(E, TK, A.device)
+    es = pre.element_size()
+    rc = lib().fx_grouped_gemm_rows_glu(ptr(A), A.stride(0), ptr(w_up), K, w_up.stride(0), 1, F * K, ptr(pre),
+                                        pre.data_ptr() + F * es, pre.stride(0), ptr(act), act.stride(0),
+                                        _counts_ptr(counts, E), E, TK, F, K, 0, dtype_enum(A.dtype), ptr(ws), nbytes,
+                                        stream_ptr(A.device))
+    check(rc, "fx_grouped_gemm_rows_glu")
+    return pre, act
+
+
+_ACT_ENUM = {"silu": 0, "gelu_tanh": 1}
+
+
+def dual_glu_supported(A, B1, B2, P1, P2, act):
+    """Whether :func:`flextrain_gemm_dual_glu` can take these tensors."""
+    if A.dtype not in (torch.bfloat16, torch.float16) or any(t.dtype != A.dtype for t in (B1, B2, P1, P2, act)):
+        return False
+    if A.dim() != 2 or B1.dim() != 2 or B1.shape != B2.shape or B1.stride() != B2.stride():
+        return False
+    if not (B1.stride(1) == 1 or B1.stride(0) == 1):
+        return False
+    K, N = B1.shape
+    ldb = B1.stride(0) if B1.stride(1) == 1 else B1.stride(1)
+    return (K % 64 == 0 and N % 8 == 0 and ldb % 8 == 0 and A.stride(1) == 1 and A.stride(0) % 8 == 0
+            and all(t.stride(1) == 1 and t.stride(0) % 8 == 0 for t in (P1, P2, act)) and P1.stride(0) == P2.stride(0)
+            and all(t.data_ptr() % 16 == 0 for t in (A, B1, B2, P1, P2, act)))
+
+
+def flextrain_gemm_dual_glu(A, B1, B2, P1, P2, act, activation="silu", gate_first=True):
+    """``P1 = A @ B1``, ``P2 = A @ B2`` and ``act = f(gate) * value`` in one launch, where
+    ``(gate, value) = (P1, P2)`` when ``gate_first``; ``B1`` / ``B2`` are ``(K, N)`` in either memory
+    order (the same for both)."""
+    M, K = A.shape
+    N = B1.shape[1]
+    if B1.shape[0] != K or tuple(P1.shape) != (M, N) or tuple(P2.shape) != (M, N) or tuple(act.shape) != (M, N):
+        raise ValueError("shape mismatch")
+    trans_b, ldb = _b_layout(B1)
+    rc = lib().fx_gemm_dual_glu(ptr(A), A.stride(0), ptr(B1), ptr(B2), ldb, trans_b, ptr(P1), ptr(P2), P1.stride(0),
+                                ptr(act), act.stride(0), M, N, K, 1 if gate_first else 0, _ACT_ENUM[activation],
+                                dtype_enum(A.dtype), stream_ptr(A.device))
+    check(rc, "fx_gemm_dual_glu")
+    return act

@@ -250,6 +250,27 @@ int fx_grouped_gemm_wgrad(const void* A, int64_t lda, const void* B, int64_t ldb
                           int M, int N, float alpha, float beta, int dt, void* ws, size_t ws_bytes,
                           hipStream_t stream);
 
+/* The expert up-projection with the SwiGLU fused into its epilogue: one launch for the GEMM of
+ * flextrain/ops/full_moe.py:428-447 and the activation kernel that follows it (:448-455).
+ * B[e] holds two halves of Nh rows (trans_b = 1, (2*Nh, K) row-major) or Nh columns (trans_b = 0),
+ * b2_delta elements apart.  P1 / P2 (row stride ldp) receive the two pre-activation halves,
+ * act (rows, Nh) = silu(gate) * value with gate = P1 when gate_first else P2, computed from the
+ * rounded P values.  Needs K % 64 == 0 and Nh % 8 == 0. */
+int fx_grouped_gemm_rows_glu(const void* A, int64_t lda, const void* B, int64_t ldb, int64_t b_expert_stride,
+                             int trans_b, int64_t b2_delta, void* P1, void* P2, int64_t ldp, void* act,
+                             int64_t ldact, const int32_t* counts, int E, int64_t total_rows, int Nh, int K,
+                             int gate_first, int dt, void* ws, size_t ws_bytes, hipStream_t stream);
+
+/* Gate and up projections of the dense gated FFN with the activation in the epilogue: replaces the
+ * two matmuls and the gated-activation launch of flextrain/nn/blocks/ffn_dense.py:130-146.
+ *   P1 = A @ op(B1), P2 = A @ op(B2) (both (M, Nh), row stride ldp), act = f(gate) * value
+ * with (gate, value) = (P1, P2) when gate_first, else (P2, P1); activation 0 = SiLU,
+ * 1 = GELU-tanh.  trans_b = 1: B are (Nh, K) row-major; 0: (K, Nh) row-major; both share ldb.
+ * Needs K % 64 == 0 and Nh % 8 == 0. */
+int fx_gemm_dual_glu(const void* A, int64_t lda, const void* B1, const void* B2, int64_t ldb, int trans_b,
+                     void* P1, void* P2, int64_t ldp, void* act, int64_t ldact, int M, int Nh, int K,
+                     int gate_first, int activation, int dt, hipStream_t stream);
+
 /* ---- GEMM dispatcher (verbatim ABI of the reference helper) --------------- */
 
 /* helpers/matmul_dispatcher/src/dispatch.h:12-35.  D = alpha*op(A)*op(B) + beta*C,
