@@ -49,7 +49,7 @@ def _parse():
     ap.add_argument("--no-extra", action="store_true", help="skip the non-headline configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--only", default="", help="comma-separated subset of the non-headline configurations "
-                                               "(c1, c3, c4, c5, ffn) to run, e.g. for a profiler pass")
+                                               "(c1, c3, c4, c5, ffn, act) to run, e.g. for a profiler pass")
     return ap.parse_args()
 
 
@@ -117,6 +117,8 @@ def run_extra(torch, ops, dev, stream, rn, only):
         rows += run_moe(torch, dev, stream, rn)
     if want("ffn"):
         rows += run_ffn_dense(torch, dev, stream, rn)
+    if want("act"):
+        rows += run_activation_slots(torch, dev)
     return rows
 
 
@@ -313,6 +315,70 @@ def run_lm_head(torch, dev, stream, rn):
     del w, g_store, logits, x, x0
     torch.cuda.empty_cache()
     return rows
+
+
+def run_activation_slots(torch, dev):
+    """Activation-slot streaming of one Llama-3.1-8B-shaped decoder layer at save level 3 (every
+    saved tensor of 8192 tokens): send_home from the HBM ring into a pinned home slot, fetch_home
+    back, and both at once on the outbound / inbound streams.  The host link is the roof."""
+    from flextrain_amd.activation_schema import ActivationField, ActivationSchema, ActivationSlot, fetch_home, send_home
+    from flextrain_amd.host_memory import LocalPinnedHostBackend
+    from flextrain_amd.streams import StreamBundle
+
+    bf, f32 = torch.bfloat16, torch.float32
+    dims = {"d": 4096, "kv": 1024, "H": 32, "F": 14336}
+    F = ActivationField
+    schema = ActivationSchema((
+        F("x_inp", lambda T, m: (T, m["d"]), bf, 0), F("attn_norm_rstd", lambda T, m: (T, 1), f32, 0),
+        F("xk", lambda T, m: (T, m["kv"]), bf, 0), F("xv", lambda T, m: (T, m["kv"]), bf, 0),
+        F("attn_result", lambda T, m: (T, m["d"]), bf, 1), F("softmax_lse", lambda T, m: (m["H"], T), f32, 1, token_axis=1),
+        F("xq", lambda T, m: (T, m["d"]), bf, 2), F("xo", lambda T, m: (T, m["d"]), bf, 2),
+        F("ffn_norm_rstd", lambda T, m: (T, 1), f32, 0),
+        F("x1", lambda T, m: (T, m["F"]), bf, 3), F("x3", lambda T, m: (T, m["F"]), bf, 3)), max_tier=3)
+    T, level = 8192, 3
+    be = LocalPinnedHostBackend()
+    sb = StreamBundle.create(dev)
+    nbytes = schema.offloaded_bytes_at_level(T, dims, level)
+    ring = torch.empty(2 * schema.device_size_bytes(T, dims), dtype=torch.uint8, device=dev)
+    half = ring.numel() // 2
+    dev_slots = [ActivationSlot.from_buffer(schema, level, T, dims, ring[i * half:(i + 1) * half], include_nonpersistent=True)[0]
+                 for i in range(2)]
+    home_bufs = [be.allocate_tensor((schema.home_size_bytes(T, dims, level),), torch.uint8) for _ in range(2)]
+    homes = [ActivationSlot.from_buffer(schema, level, T, dims, b)[0] for b in home_bufs]
+
+    def timed(fn):
+        fn()
+        sb.synchronize_all()
+        ts = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            fn()
+            sb.synchronize_all()
+            ts.append(time.perf_counter() - t0)
+        return sorted(ts)[1] * 1e3
+
+    def out():
+        with torch.cuda.stream(sb.outbound):
+            send_home(homes[0], dev_slots[0], level)
+
+    def back():
+        with torch.cuda.stream(sb.inbound):
+            fetch_home(dev_slots[1], homes[1], level)
+
+    def both():
+        out()
+        back()
+
+    ms_out, ms_in, ms_both = timed(out), timed(back), timed(both)
+    row = {"op": "act.activation slot of one decoder layer, 8192 tokens, save level 3 (11 fields, one library call per slot)",
+           "algorithmic": nbytes, "unit": "GB/s (host link)", "frac": None,
+           "send_home_ms": round(ms_out, 3), "send_home_GBps": round(nbytes / ms_out / 1e6, 2),
+           "fetch_home_ms": round(ms_in, 3), "fetch_home_GBps": round(nbytes / ms_in / 1e6, 2),
+           "both_directions_ms": round(ms_both, 3), "both_directions_GBps_each": round(nbytes / ms_both / 1e6, 2),
+           "ms": round(ms_both, 3), "achieved": round(2 * nbytes / ms_both / 1e6, 2)}
+    for b in home_bufs:
+        be.release(b)
+    return [row]
 
 
 def run_ffn_dense(torch, dev, stream, rn):

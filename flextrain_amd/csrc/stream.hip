@@ -184,3 +184,42 @@ extern "C" int fx_host_unregister(void* ptr) {
     }
     return 0;
 }
+
+// Every field of one activation slot moved in ONE call: field i is rows[i] rows of row_bytes[i]
+// bytes, source and destination rows src_pitch[i] / dst_pitch[i] bytes apart (a pitch equal to
+// row_bytes means contiguous, and the whole field goes as one linear copy; a wider pitch is the
+// narrowed view of a tensor sized for more tokens and goes as a 2-D copy).  The reference issues
+// one torch copy_ per field (flextrain/core/activation_schema.py:483-519); batching them keeps the
+// host cost of an offload at one library call per (chunk, layer) slot.
+extern "C" int fx_copy_fields(int n, void* const* dst, const void* const* src, const int64_t* rows,
+                              const int64_t* row_bytes, const int64_t* dst_pitch, const int64_t* src_pitch,
+                              int direction, hipStream_t stream) {
+    if (n < 0) FX_FAIL("fx_copy_fields: negative field count");
+    if (n == 0) return 0;
+    if (!dst || !src || !rows || !row_bytes || !dst_pitch || !src_pitch) FX_FAIL("fx_copy_fields: null array");
+    hipMemcpyKind kind;
+    switch (direction) {
+        case 0: kind = hipMemcpyDeviceToHost; break;
+        case 1: kind = hipMemcpyHostToDevice; break;
+        case 2: kind = hipMemcpyDeviceToDevice; break;
+        default: FX_FAIL("fx_copy_fields: direction must be 0 (device to host), 1 (host to device) or 2 (device to device)");
+    }
+    for (int i = 0; i < n; ++i) {
+        if (rows[i] < 0 || row_bytes[i] < 0) FX_FAIL("fx_copy_fields: field %d has a negative extent", i);
+        if (rows[i] == 0 || row_bytes[i] == 0) continue;
+        if (!dst[i] || !src[i]) FX_FAIL("fx_copy_fields: field %d has a null pointer", i);
+        if (dst_pitch[i] < row_bytes[i] || src_pitch[i] < row_bytes[i])
+            FX_FAIL("fx_copy_fields: field %d has a pitch smaller than its row", i);
+        hipError_t e;
+        if (rows[i] == 1 || (dst_pitch[i] == row_bytes[i] && src_pitch[i] == row_bytes[i]))
+            e = hipMemcpyAsync(dst[i], src[i], (size_t)(rows[i] * row_bytes[i]), kind, stream);
+        else
+            e = hipMemcpy2DAsync(dst[i], (size_t)dst_pitch[i], src[i], (size_t)src_pitch[i], (size_t)row_bytes[i],
+                                 (size_t)rows[i], kind, stream);
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            FX_FAIL("fx_copy_fields: copy of field %d failed: %s", i, hipGetErrorString(e));
+        }
+    }
+    return 0;
+}

@@ -309,6 +309,15 @@ int fx_host_free(void* ptr);
 int fx_host_register(void* ptr, size_t bytes);
 int fx_host_unregister(void* ptr);
 
+/* send_home / fetch_home of one activation slot (flextrain/core/activation_schema.py:483-519; the
+ * engine's call sites are flextrain/engine/active_model.py:1184-1199 and :2036-2098): all n
+ * fields in one call.  Field i: rows[i] rows of row_bytes[i] bytes, rows dst_pitch[i] /
+ * src_pitch[i] bytes apart.  direction 0 = device to host, 1 = host to device, 2 = device to
+ * device.  Enqueued on `stream`, not waited for. */
+int fx_copy_fields(int n, void* const* dst, const void* const* src, const int64_t* rows,
+                   const int64_t* row_bytes, const int64_t* dst_pitch, const int64_t* src_pitch,
+                   int direction, hipStream_t stream);
+
 /* Device staging bytes fx_adamw_stream_chunk needs for n_slots slots of sub_elems
  * elements (p, g, m, v and, when stage_bf16_copy, the bf16 copy of p). */
 size_t fx_adamw_stream_ws_bytes(int64_t sub_elems, int n_slots, int p_dt, int g_dt, int state_dt,
