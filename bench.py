@@ -49,7 +49,7 @@ def _parse():
     ap.add_argument("--no-extra", action="store_true", help="skip the non-headline configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--only", default="", help="comma-separated subset of the non-headline configurations "
-                                               "(c1, c3, c4, c5, ffn, act) to run, e.g. for a profiler pass")
+                                               "(c1, c3, c4, c5, ffn, act, probe) to run, e.g. for a profiler pass")
     return ap.parse_args()
 
 
@@ -119,6 +119,8 @@ def run_extra(torch, ops, dev, stream, rn, only):
         rows += run_ffn_dense(torch, dev, stream, rn)
     if want("act"):
         rows += run_activation_slots(torch, dev)
+    if want("probe"):
+        rows += run_hw_probe(torch, dev)
     return rows
 
 
@@ -315,6 +317,19 @@ def run_lm_head(torch, dev, stream, rn):
     del w, g_store, logits, x, x0
     torch.cuda.empty_cache()
     return rows
+
+
+def run_hw_probe(torch, dev):
+    """The inputs of the save-level solver as the library's probe measures them on this box
+    (sustained GEMM rate on random operands, HBM streaming rate, concurrent host-link rate)."""
+    from flextrain_amd.hw_probe import probe_hardware
+
+    r = probe_hardware(device=dev, matmul_target_seconds=3.0, mem_bw_target_seconds=1.0)
+    return [{"op": "probe.save-level solver inputs (8192^3 bf16 GEMM, two-half sustained window)", "algorithmic": None,
+             "ms": round(r.matmul_per_call_ms, 4), "achieved": round(r.achieved_tflops_second_half, 1), "unit": "TFLOP/s",
+             "frac": round(r.achieved_tflops_second_half / BF16_PEAK_TFLOPS, 4),
+             "tflops_first_half": round(r.achieved_tflops_first_half, 1), "hbm_stream_GBps": round(r.mem_bw_gbps, 1),
+             "host_link_GBps_each_direction_concurrent": round(r.hw_cost.pcie_bw_gbps, 2)}]
 
 
 def run_activation_slots(torch, dev):
