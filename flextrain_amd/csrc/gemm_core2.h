@@ -310,8 +310,32 @@ FX_DEV void epilogue_tile(f32x16_t (&acc)[WM / 32][WN / 32], const TD* C, TD* D,
     float* stage = reinterpret_cast<float*>(smem) + wave * 32 * PITCH;
     const bool vec_ok = ((ldd & 7) == 0) && ((reinterpret_cast<uintptr_t>(D) & 15u) == 0) &&
                         (beta == 0.f || (((ldc & 7) == 0) && ((reinterpret_cast<uintptr_t>(C) & 15u) == 0)));
+    // With beta != 0 the C values of several bands are fetched together before the bands are
+    // staged: one exposed memory round trip per group instead of one per band and lane slot (a
+    // short-K tile spends as long in its epilogue as in its K loop otherwise).  A group is as many
+    // bands as fit 64 registers per lane.
+    typedef typename VecOf<TD>::type CV;
+    constexpr int CVN = 8 / VecOf<TD>::N;                                   // 16-byte vectors per 8 elements
+    constexpr int CB = (CVN == 1 || TM == 1) ? TM : TM / 2;                 // bands per prefetch group
+    static_assert(TM % CB == 0, "bands must split evenly into prefetch groups");
+    CV cpre[CB][PER_LANE][CVN];
+    const bool pre_c = vec_ok && beta != 0.f;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
+        if (pre_c && i % CB == 0) {
+#pragma unroll
+            for (int b = 0; b < CB; ++b)
+#pragma unroll
+                for (int t = 0; t < PER_LANE; ++t) {
+                    const int id = t * 64 + lane;
+                    const int row = row_base + (i + b) * 32 + id / GROUPS, col = col_base + (id % GROUPS) * 8;
+                    if (row < M && col + 8 <= N) {
+#pragma unroll
+                        for (int q = 0; q < CVN; ++q)
+                            cpre[b][t][q] = *reinterpret_cast<const CV*>(C + (int64_t)row * ldc + col + q * VecOf<TD>::N);
+                    }
+                }
+        }
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
@@ -334,10 +358,11 @@ FX_DEV void epilogue_tile(f32x16_t (&acc)[WM / 32][WN / 32], const TD* C, TD* D,
             TD* dst = D + (int64_t)row * ldd + col;
             if (vec_ok && col + 8 <= N) {
                 if (beta != 0.f) {
-                    float c[8];
-                    load_f32<TD, 8>(C + (int64_t)row * ldc + col, c);
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) o[e] += beta * c[e];
+                    for (int q = 0; q < CVN; ++q)
+#pragma unroll
+                        for (int e = 0; e < VecOf<TD>::N; ++e)
+                            o[q * VecOf<TD>::N + e] += beta * (float)cpre[i % CB][t][q][e];
                 }
                 store_f32<TD, 8>(dst, o);
             } else {
