@@ -90,9 +90,9 @@ static TileCfg choose_tile(int M, int N) {
 // 1024 x 4096 with K = 128256): the largest tile, K cut into `splits` ranges of a multiple of 64.
 static int choose_splits(int M, int N, int K, size_t workspace_bytes) {
     const long tiles = (long)cdiv(M, 256) * cdiv(N, 256);
-    if (tiles >= 128 || K < 4096) return 1;
+    if (tiles >= 128 || K < 1024) return 1;
     long s = 256 / tiles;
-    if (s > K / 2048) s = K / 2048;
+    if (s > K / 512) s = K / 512;       // at least 8 K-steps per split
     const size_t per = (size_t)M * N * sizeof(float);
     if (per == 0 || (size_t)s * per > workspace_bytes) s = (long)(workspace_bytes / (per ? per : 1));
     if (s > 16) s = 16;
