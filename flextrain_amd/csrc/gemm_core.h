@@ -55,9 +55,9 @@ struct OperandView {
     int ext;
     int origin;
     // Two-matrix tile (loaders instantiated with DUAL): tile rows >= half come from the matrix
-    // that starts half_delta elements after `base`, at index origin + row - half.
+    // at `base2` (same ld and extent), at index origin + row - half.
     int half = 0;
-    int64_t half_delta = 0;
+    const T* base2 = nullptr;
 };
 
 // Registers that park one K-step of one operand tile (ROWS x 64 elements):

@@ -53,9 +53,7 @@ FX_DEV void tile_load_direct(const OperandView<T>& op, int k0, T* lds, int wave,
         int g = op.origin + (second ? r - op.half : r);
         g = g < op.ext ? g : op.ext - 1;
         const int c = pos ^ swz(r);
-        const T* src = op.base + (int64_t)g * op.ld + k0 + c * 8;
-        if (second) src += op.half_delta;
-        load_to_lds16(src, lds + (j * NW + wave) * 8 * GEMM_BK);
+        load_to_lds16((second ? op.base2 : op.base) + (int64_t)g * op.ld + k0 + c * 8, lds + (j * NW + wave) * 8 * GEMM_BK);
     }
 }
 
@@ -78,9 +76,7 @@ FX_DEV void tile_load_direct_tr(const OperandView<T>& op, int k0, T* lds, int wa
         const bool second = DUAL && c * 8 >= op.half;
         int g = op.origin + (second ? c * 8 - op.half : c * 8);
         g = g + 8 <= op.ext ? g : op.ext - 8;
-        const T* src = op.base + (int64_t)(k0 + k) * op.ld + g;
-        if (second) src += op.half_delta;
-        load_to_lds16(src, lds + q * 512);
+        load_to_lds16((second ? op.base2 : op.base) + (int64_t)(k0 + k) * op.ld + g, lds + q * 512);
     }
 }
 

@@ -12,13 +12,13 @@ namespace fx {
 
 template <typename T, bool B_MN, int ACT>
 __global__ __launch_bounds__(512) void gemm_dual_glu_kernel(
-    const T* __restrict__ A, int64_t lda, const T* __restrict__ B1, int64_t b2_delta, int64_t ldb, T* P1, T* P2,
+    const T* __restrict__ A, int64_t lda, const T* __restrict__ B1, const T* __restrict__ B2, int64_t ldb, T* P1, T* P2,
     int64_t ldp, T* ACTO, int64_t ldact, int M, int Nh, int K, int gate_first, int tiles_m, int tiles_n) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     int tm, tn;
     tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
     OperandView<T> a{A, lda, M, tm * 256};
-    OperandView<T> b{B1, ldb, Nh, tn * 128, 128, b2_delta};
+    OperandView<T> b{B1, ldb, Nh, tn * 128, 128, B2};
     gemm_tile2_glu<T, 256, 256, 2, 4, B_MN, ACT>(a, b, P1, P2, ldp, ACTO, ldact, M, Nh, K, gate_first != 0,
                                                  reinterpret_cast<T*>(smem_raw));
 }
@@ -34,9 +34,8 @@ static void launch_dual(const void* A, int64_t lda, const void* B1, const void* 
         attr_set = true;
     }
     const int tiles_m = (M + 255) / 256, tiles_n = (Nh + 127) / 128;
-    const int64_t delta = reinterpret_cast<const T*>(B2) - reinterpret_cast<const T*>(B1);
     kern<<<dim3((unsigned)(tiles_m * tiles_n)), 512, lds, s>>>(
-        reinterpret_cast<const T*>(A), lda, reinterpret_cast<const T*>(B1), delta, ldb, reinterpret_cast<T*>(P1),
+        reinterpret_cast<const T*>(A), lda, reinterpret_cast<const T*>(B1), reinterpret_cast<const T*>(B2), ldb, reinterpret_cast<T*>(P1),
         reinterpret_cast<T*>(P2), ldp, reinterpret_cast<T*>(act), ldact, M, Nh, K, gate_first, tiles_m, tiles_n);
 }
 
@@ -52,10 +51,8 @@ extern "C" int fx_gemm_dual_glu(const void* A, int64_t lda, const void* B1, cons
     if (!A || !B1 || !B2 || !P1 || !P2 || !act) FX_FAIL("fx_gemm_dual_glu: null pointer");
     if (dt != DT_BF16 && dt != DT_F16) FX_FAIL("fx_gemm_dual_glu: bf16 or fp16 only");
     if (activation != ACT_SILU && activation != ACT_GELU_TANH) FX_FAIL("fx_gemm_dual_glu: unknown activation %d", activation);
-    const size_t es = 2;
     if ((K & 63) || (Nh & 7) || (lda & 7) || (ldb & 7) || (ldp & 7) || (ldact & 7) || !aligned16(A) || !aligned16(B1) ||
-        !aligned16(B2) || !aligned16(P1) || !aligned16(P2) || !aligned16(act) ||
-        ((reinterpret_cast<uintptr_t>(B2) - reinterpret_cast<uintptr_t>(B1)) % es) != 0)
+        !aligned16(B2) || !aligned16(P1) || !aligned16(P2) || !aligned16(act))
         FX_FAIL("fx_gemm_dual_glu: needs K %% 64 == 0, N %% 8 == 0, leading dimensions %% 8 == 0 and 16-byte aligned operands");
 #define FX_DUAL(TT)                                                                                           \
     {                                                                                                         \

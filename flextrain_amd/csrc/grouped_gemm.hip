@@ -116,7 +116,8 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void grouped_rows_glu_kerne
     const int64_t row0 = OFFSETS[e];
     const int rows = OFFSETS[e + 1] - OFFSETS[e];
     OperandView<T> a{A + row0 * lda, lda, rows, m0};
-    OperandView<T> b{B + (int64_t)e * b_expert_stride, ldb, Nh, tn * (BN / 2), BN / 2, b2_delta};
+    const T* b1 = B + (int64_t)e * b_expert_stride;
+    OperandView<T> b{b1, ldb, Nh, tn * (BN / 2), BN / 2, b1 + b2_delta};
     gemm_tile2_glu<T, BM, BN, WAVES_M, WAVES_N, B_MN, ACT_SILU>(a, b, P1 + row0 * ldp, P2 + row0 * ldp, ldp,
                                                                 ACTO + row0 * ldact, ldact, rows, Nh, K,
                                                                 gate_first != 0, smem);
