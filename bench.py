@@ -611,7 +611,7 @@ def main():
         cpu_step()
         times = []
         t_begin = time.perf_counter()
-        while len(times) < 3 or (time.perf_counter() - t_begin < 10.0 and len(times) < 50):
+        while len(times) < 3 or (time.perf_counter() - t_begin < 12.0 and len(times) < 400):  # about 12 s of CPU work
             t1 = time.perf_counter()
             cpu_step()
             times.append(time.perf_counter() - t1)
