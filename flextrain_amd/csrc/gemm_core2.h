@@ -220,7 +220,10 @@ FX_DEV void mma_step(const T* As, const T* Bs, int row_a0, int row_b0, int lane,
 // one K-step can run after the workgroup barrier while the first fragments of the next K-step are
 // being read.  Without that, every K-step starts with the matrix pipe idle for the LDS latency of
 // eight waves' first reads.
-template <typename T, int BM, int BN, int WM, int WN, bool A_TR, bool B_TR>
+// Swizzle of a K-contiguous tile whose rows hold BK k-values: 8 chunks per row (BK = 64) or 4 (BK = 32).
+template <int BK> FX_DEV int swz_k(int r) { return BK == 64 ? swz(r) : ((r >> 2) & 3); }
+
+template <typename T, int BM, int BN, int WM, int WN, bool A_TR, bool B_TR, int BK = GEMM_BK>
 struct MmaPipe {
     static constexpr int TM = WM / 32, TN = WN / 32;
     static constexpr int READS = TM + TN, MFMAS = TM * TN;
@@ -236,7 +239,7 @@ struct MmaPipe {
 
     static FX_DEV frag read_k(const T* base, int row0, int ks, int lane) {
         const int r = row0 + (lane & 31);
-        return *reinterpret_cast<const frag*>(base + r * GEMM_BK + (((ks * 2 + (lane >> 5)) ^ swz(r)) << 3));
+        return *reinterpret_cast<const frag*>(base + r * BK + (((ks * 2 + (lane >> 5)) ^ swz_k<BK>(r)) << 3));
     }
     static FX_DEV frag read_tr(const T* base, int pitch, int col0, int ks, int lane) {
         const int grp = lane >> 4, sl = lane & 15;
@@ -534,6 +537,116 @@ FX_DEV void gemm_tile2_glu(const OperandView<T>& A, const OperandView<T>& B, T* 
         }
         __syncthreads();
     }
+}
+
+// ---------------------------------------------------------------- 32-wide K-steps, three LDS stages
+// For problems whose tiles are short-lived (grouped expert GEMMs: K of a few hundred to 2048, a
+// large epilogue per tile) the K loop also exists with 32-wide steps: a 128 x 256 (or 256 x 128)
+// tile of four waves needs 24 KB per stage, three stages fit the LDS twice per CU, and with at
+// most 256 registers per lane two workgroups share a CU: one's epilogue and prologue overlap the
+// other's K loop, and the loads of two K-steps are in flight instead of one.
+//   K-contiguous tile: LDS row r holds 32 k-values as four 16-byte chunks, chunk c at position
+//     c ^ ((r >> 2) & 3) (16 consecutive rows of one chunk column hit 64 distinct banks); a wave
+//     instruction covers 16 rows.
+//   M/N-contiguous tile: as in the 64-wide form (row k holds the tile's m or n values), 32 rows.
+template <typename T, int ROWS, int NW>
+FX_DEV void tile32_load_direct(const OperandView<T>& op, int k0, T* lds, int wave, int lane) {
+    constexpr int NI = ROWS / 16 / NW;
+    static_assert(ROWS % (16 * NW) == 0, "tile rows must split evenly over the waves");
+    const int rr = lane >> 2, pos = lane & 3;
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+        const int r = (j * NW + wave) * 16 + rr;
+        int g = op.origin + r;
+        g = g < op.ext ? g : op.ext - 1;
+        const int c = pos ^ swz_k<32>(r);
+        load_to_lds16(op.base + (int64_t)g * op.ld + k0 + c * 8, lds + (j * NW + wave) * 16 * 32);
+    }
+}
+
+template <typename T, int ROWS, int NW>
+FX_DEV void tile32_load_direct_tr(const OperandView<T>& op, int k0, T* lds, int wave, int lane) {
+    constexpr int CPR = ROWS / 8;               // 16-byte chunks per LDS row
+    constexpr int KPI = 64 / CPR;               // k-rows per instruction
+    constexpr int NI = 32 / KPI / NW;           // instructions per wave
+    static_assert((ROWS == 128 || ROWS == 256) && (32 / KPI) % NW == 0, "unsupported tile rows");
+    const int kin = lane / CPR, pos = lane % CPR;
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+        const int q = j * NW + wave;
+        const int k = q * KPI + kin;
+        const int c = pos ^ (swz_tr(k) % CPR);
+        int g = op.origin + c * 8;
+        g = g + 8 <= op.ext ? g : op.ext - 8;
+        load_to_lds16(op.base + (int64_t)(k0 + k) * op.ld + g, lds + q * 512);
+    }
+}
+
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N>
+constexpr size_t gemm32_lds_bytes() {
+    constexpr size_t tiles = (size_t)3 * (BM + BN) * 32 * sizeof(T);
+    constexpr size_t epi = epilogue_lds_bytes<WAVES_M * WAVES_N, BN / WAVES_N>();
+    return tiles > epi ? tiles : epi;
+}
+
+// K loop with 32-wide steps over three rotating LDS stages; K must be a multiple of 32.
+// Leaves the accumulators in `acc` and ends with a barrier (the stages become epilogue staging).
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_MN, bool B_MN>
+FX_DEV void gemm_mainloop32(const OperandView<T>& A, const OperandView<T>& B, int K, T* smem,
+                            f32x16_t (&acc)[BM / WAVES_M / 32][BN / WAVES_N / 32]) {
+    constexpr int NW = WAVES_M * WAVES_N;
+    constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+    constexpr int TM = WM / 32, TN = WN / 32;
+    constexpr int STAGE = (BM + BN) * 32;
+    constexpr int LD = (BM + BN) * 64 / 1024 / NW;      // load instructions per wave per K-step
+    static_assert((BM + BN) * 64 % (1024 * NW) == 0, "loads must split evenly over the waves");
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+    const int n = K / 32;
+    auto issue = [&](int kt, T* buf) {
+        if (!A_MN) tile32_load_direct<T, BM, NW>(A, kt * 32, buf, wave, lane);
+        else tile32_load_direct_tr<T, BM, NW>(A, kt * 32, buf, wave, lane);
+        if (!B_MN) tile32_load_direct<T, BN, NW>(B, kt * 32, buf + BM * 32, wave, lane);
+        else tile32_load_direct_tr<T, BN, NW>(B, kt * 32, buf + BM * 32, wave, lane);
+    };
+    if (n > 0) {
+        typedef MmaPipe<T, BM, BN, WM, WN, A_MN, B_MN, 32> Pipe;
+        typename Pipe::Slot f0, f1;
+        const int ra = wm * WM, rb = wn * WN;
+        T* cur = smem;
+        T* nxt = smem + STAGE;
+        T* aft = smem + 2 * STAGE;
+        issue(0, cur);
+        if (n > 1) {
+            issue(1, nxt);
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LD) : "memory");   // step 0 landed, step 1 may be in flight
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+        __syncthreads();
+        if (n > 2) issue(2, aft);
+        Pipe::fetch_all(f0, cur, cur + BM * 32, 0, ra, rb, lane);
+        for (int kt = 0; kt + 1 < n; ++kt) {
+            Pipe::template sub<true>(acc, f0, f1, cur, cur + BM * 32, 1, ra, rb, lane);
+            // every read of `cur` is issued; step kt+1 must have landed (step kt+2 may still fly)
+            if (kt + 2 < n) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(LD) : "memory");
+            else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+            __syncthreads();
+            if (kt + 3 < n) issue(kt + 3, cur);          // `cur` is free for everyone now
+            Pipe::template sub<true>(acc, f1, f0, nxt, nxt + BM * 32, 0, ra, rb, lane);
+            T* t = cur; cur = nxt; nxt = aft; aft = t;
+        }
+        Pipe::template sub<true>(acc, f0, f1, cur, cur + BM * 32, 1, ra, rb, lane);
+        Pipe::template sub<false>(acc, f1, f0, cur, cur, 0, ra, rb, lane);
+    }
+    __syncthreads();
+    static_assert(gemm32_lds_bytes<T, BM, BN, WAVES_M, WAVES_N>() <= 80 * 1024, "two workgroups must fit the LDS of a CU");
 }
 
 // ---------------------------------------------------------------- workgroup -> tile maps

@@ -43,7 +43,9 @@ def _ragged_counts(g, E, TK):
     return c
 
 
-@pytest.mark.parametrize("E,TK,K,N", [(8, 1000, 256, 384), (128, 65536, 2048, 1536), (4, 300, 64, 72), (3, 50, 8, 8)])
+@pytest.mark.parametrize("E,TK,K,N", [(8, 1000, 256, 384), (128, 65536, 2048, 1536), (4, 300, 64, 72), (3, 50, 8, 8),
+                                      (5, 700, 96, 520),       # K a multiple of 32 only, N not a multiple of the tile
+                                      (3, 5000, 160, 264)])    # large experts: 256-row tiles, K tail of 32
 @pytest.mark.parametrize("trans_b", [True, False])
 def test_grouped_rows(dev, E, TK, K, N, trans_b):
     g = gen(E * 13 + N)
