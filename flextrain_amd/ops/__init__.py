@@ -32,6 +32,7 @@ from .softmax_ce import (
     flextrain_cross_entropy_loss,
     flextrain_softmax,
     flextrain_softmax_cross_entropy,
+    flextrain_softmax_cross_entropy_loss,
 )
 from .rope import (
     build_rope_inv_freq,
@@ -90,6 +91,7 @@ __all__ = [
     "flextrain_rope_partial_fwd",
     "flextrain_softmax",
     "flextrain_softmax_cross_entropy",
+    "flextrain_softmax_cross_entropy_loss",
     "flextrain_swiglu_bwd",
     "flextrain_swiglu_fwd",
 ]

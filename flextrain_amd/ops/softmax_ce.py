@@ -96,6 +96,32 @@ def flextrain_cross_entropy_loss(P_in, labels, L=None, Valid_Count_out=None, max
     return P_in, L
 
 
+def flextrain_softmax_cross_entropy_loss(X, labels, L=None, Valid_Count=None):
+    """The reference's summary wrapper (flextrain/ops/_kernels/cross_entropy.py:215-268): runs the
+    probability cross-entropy kernel on ``X`` in place (``X`` becomes ``P - onehot``, rows with a
+    negative label become zero), then reduces on the device and returns
+    ``(X, L, total_loss, avg_loss, num_valid_labels)`` with the three scalars as Python floats
+    (this synchronises with the host, as the reference's ``.item()`` calls do)."""
+    T, V = X.shape
+    assert X.is_contiguous(), "Input tensor X must be contiguous"
+    assert labels.shape == (T,), f"Labels tensor must have shape ({T},), but got {labels.shape}"
+    if L is not None:
+        assert L.shape == (T,), f"L must have shape {(T,)}, but got {L.shape}"
+        assert L.device == X.device, "L must be on the same device as X"
+        assert L.dtype == torch.float32, "L must be dtype torch.float32"
+    if Valid_Count is None:
+        Valid_Count = torch.empty((T,), dtype=torch.float32, device=X.device)
+    else:
+        assert Valid_Count.shape == (T,), f"Valid_Count must have shape {(T,)}, but got {Valid_Count.shape}"
+        assert Valid_Count.device == X.device, "Valid_Count must be on the same device as X"
+        assert Valid_Count.dtype == torch.float32, "Valid_Count must be dtype torch.float32"
+    X, L = flextrain_cross_entropy_loss(X, labels, L=L, Valid_Count_out=Valid_Count)
+    total_loss = torch.sum(L)
+    num_valid_labels = torch.sum(Valid_Count)
+    avg_loss = total_loss / (num_valid_labels + 1e-8)
+    return X, L, total_loss.item(), avg_loss.item(), num_valid_labels.item()
+
+
 def flextrain_softmax_cross_entropy(logits, labels, L=None, dZ=None, loss_mask=None, max_idx_out=None,
                                     max_val_out=None, ignore_index=-100, max_loss=100.0):
     """Fused row softmax + cross-entropy + dZ.  ``dZ`` defaults to ``logits`` (in

@@ -65,6 +65,13 @@ def test_cross_entropy_from_probs_in_place(dev, dtype):
     pd2 = p.to(dev)
     _, loss2 = ops.flextrain_cross_entropy_loss(pd2, labels.to(torch.int32).to(dev))
     assert torch.equal(loss2, loss) and torch.equal(pd2, pd)
+    # the summary wrapper: same kernel, then the three scalars on the host
+    pd3 = p.to(dev)
+    X, L, total, avg, n_valid = ops.flextrain_softmax_cross_entropy_loss(pd3, labels.to(dev))
+    assert X.data_ptr() == pd3.data_ptr() and torch.equal(pd3, pd) and torch.equal(L, loss)
+    assert n_valid == float(valid_ref.sum()) and isinstance(total, float)
+    assert total == pytest.approx(float(loss_ref.sum()), rel=1e-5)
+    assert avg == pytest.approx(float(loss_ref.sum()) / float(valid_ref.sum()), rel=1e-5)
 
 
 @pytest.mark.parametrize("T,V", [(40, 128256), (9, 777), (16, 4096)])
