@@ -45,6 +45,7 @@ def _ragged_counts(g, E, TK):
 
 @pytest.mark.parametrize("E,TK,K,N", [(8, 1000, 256, 384), (128, 65536, 2048, 1536), (4, 300, 64, 72), (3, 50, 8, 8),
                                       (5, 700, 96, 520),       # K a multiple of 32 only, N not a multiple of the tile
+                                      (3, 200, 32, 40),        # a single 32-wide K-step
                                       (3, 5000, 160, 264)])    # large experts: 256-row tiles, K tail of 32
 @pytest.mark.parametrize("trans_b", [True, False])
 def test_grouped_rows(dev, E, TK, K, N, trans_b):
@@ -72,6 +73,21 @@ def test_grouped_rows(dev, E, TK, K, N, trans_b):
     a, b = int(off[e]), int(off[e + 1])
     Be = W[e].float().t() if trans_b else W[e].float()
     _close_scaled(D2[a:b], 0.5 * (A[a:b].float() @ Be) + C[a:b].float(), "beta path")
+
+
+def test_grouped_rows_fp16(dev):
+    g = gen(77)
+    E, TK, K, N = 6, 900, 128, 200
+    counts = _ragged_counts(g, E, TK)
+    A = randn(g, TK, K, std=0.5, dtype=torch.float16)
+    W = randn(g, E, N, K, std=0.1, dtype=torch.float16)
+    D = torch.empty((TK, N), dtype=torch.float16, device=dev)
+    flextrain_grouped_gemm_rows(A.to(dev), W.to(dev).transpose(1, 2), counts.to(dev), D)
+    off = o_moe.expert_offsets(counts)
+    for e in range(E):
+        a, b = int(off[e]), int(off[e + 1])
+        if a < b:
+            _close_scaled(D[a:b], A[a:b].float() @ W[e].float().t(), f"expert {e}")
 
 
 @pytest.mark.parametrize("E,TK,M,N", [(8, 1000, 256, 384), (128, 65536, 1536, 2048), (4, 300, 64, 72)])
