@@ -134,6 +134,20 @@ constexpr size_t kStreamingBytes = (size_t)96 << 20;
 
 inline int elem_size(int dt) { return dt == DT_F32 ? 4 : 2; }
 
+// More than 64 KB of dynamic LDS has to be asked for, once per kernel AND device.  One bit per
+// device at each call site; racing host threads at worst repeat the (idempotent) call.
+#define FX_ENSURE_DYNAMIC_LDS(kern, bytes)                                                          \
+    do {                                                                                           \
+        static unsigned long long done__ = 0ull;                                                   \
+        int dev__ = 0;                                                                             \
+        (void)hipGetDevice(&dev__);                                                                \
+        if (dev__ < 0 || dev__ >= 64 || !((done__ >> dev__) & 1ull)) {                             \
+            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                         \
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)(bytes));   \
+            if (dev__ >= 0 && dev__ < 64) done__ |= 1ull << dev__;                                 \
+        }                                                                                          \
+    } while (0)
+
 #define FX_CHECK_LAUNCH(name)                                                        \
     do {                                                                             \
         hipError_t e__ = hipGetLastError();                                          \

@@ -104,11 +104,7 @@ static void launch_one(const T* a, const T* b, const TD* c, TD* d, float* part, 
                        int64_t lda, int64_t ldb, int64_t ldc, int64_t ldd, float alpha, float beta, hipStream_t s) {
     auto kern = gemm_kernel<T, TD, BM, BN, WAVES_M, WAVES_N, A_MN, B_MN>;
     constexpr size_t lds = gemm2_lds_bytes<T, BM, BN, WAVES_M, WAVES_N>();
-    static bool attr_set = false;  // more than 64 KB of dynamic LDS has to be asked for once per kernel
-    if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        attr_set = true;
-    }
+    FX_ENSURE_DYNAMIC_LDS(kern, lds);
     const int tiles_m = cdiv(M, BM), tiles_n = cdiv(N, BN);
     int k_per_split = K;
     if (splits > 1) k_per_split = cdiv(cdiv(K, splits), GEMM_BK) * GEMM_BK;

@@ -28,11 +28,7 @@ static void launch_dual(const void* A, int64_t lda, const void* B1, const void* 
                         int64_t ldp, void* act, int64_t ldact, int M, int Nh, int K, int gate_first, hipStream_t s) {
     auto kern = gemm_dual_glu_kernel<T, B_MN, ACT>;
     constexpr size_t lds = gemm2_lds_bytes<T, 256, 256, 2, 4>();
-    static bool attr_set = false;  // more than 64 KB of dynamic LDS has to be asked for once per kernel
-    if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        attr_set = true;
-    }
+    FX_ENSURE_DYNAMIC_LDS(kern, lds);
     const int tiles_m = (M + 255) / 256, tiles_n = (Nh + 127) / 128;
     kern<<<dim3((unsigned)(tiles_m * tiles_n)), 512, lds, s>>>(
         reinterpret_cast<const T*>(A), lda, reinterpret_cast<const T*>(B1), reinterpret_cast<const T*>(B2), ldb, reinterpret_cast<T*>(P1),

@@ -214,12 +214,7 @@ extern "C" int fx_grouped_gemm_rows(const void* A, int64_t lda, const void* B, i
     {                                                                                                     \
         auto kern = grouped_rows_kernel<TT, BM_, BN_, WM_, WN_, BMN>;                                     \
         constexpr size_t lds = gemm2_lds_bytes<TT, BM_, BN_, WM_, WN_>();                                 \
-        static bool attr_set = false;                                                                     \
-        if (!attr_set) {                                                                                  \
-            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                \
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);              \
-            attr_set = true;                                                                              \
-        }                                                                                                 \
+        FX_ENSURE_DYNAMIC_LDS(kern, lds);                                                                 \
         const int tiles_n = cdiv_i(N, BN_);                                                               \
         kern<<<dim3(max_tiles * (unsigned)tiles_n), WM_ * WN_ * 64, lds, stream>>>(                       \
             reinterpret_cast<const TT*>(A), lda, reinterpret_cast<const TT*>(B), ldb, b_expert_stride,    \
@@ -230,12 +225,7 @@ extern "C" int fx_grouped_gemm_rows(const void* A, int64_t lda, const void* B, i
     {                                                                                                     \
         auto kern = grouped_rows_kernel32<TT, 128, 256, 2, 2, BMN>;                                       \
         constexpr size_t lds = gemm32_lds_bytes<TT, 128, 256, 2, 2>();                                    \
-        static bool attr_set = false;                                                                     \
-        if (!attr_set) {                                                                                  \
-            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                \
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);              \
-            attr_set = true;                                                                              \
-        }                                                                                                 \
+        FX_ENSURE_DYNAMIC_LDS(kern, lds);                                                                 \
         const int tiles_n = cdiv_i(N, 256);                                                               \
         kern<<<dim3(max_tiles * (unsigned)tiles_n), 256, lds, stream>>>(                                  \
             reinterpret_cast<const TT*>(A), lda, reinterpret_cast<const TT*>(B), ldb, b_expert_stride,    \
@@ -279,12 +269,7 @@ extern "C" int fx_grouped_gemm_rows_glu(const void* A, int64_t lda, const void* 
     {                                                                                                     \
         auto kern = grouped_rows_glu_kernel<TT, BM_, BN_, WM_, WN_, BMN>;                                 \
         constexpr size_t lds = gemm2_lds_bytes<TT, BM_, BN_, WM_, WN_>();                                 \
-        static bool attr_set = false;                                                                     \
-        if (!attr_set) {                                                                                  \
-            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                \
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);              \
-            attr_set = true;                                                                              \
-        }                                                                                                 \
+        FX_ENSURE_DYNAMIC_LDS(kern, lds);                                                                 \
         const int tiles_n = cdiv_i(Nh, BN_ / 2);                                                          \
         kern<<<dim3(max_tiles * (unsigned)tiles_n), WM_ * WN_ * 64, lds, stream>>>(                       \
             reinterpret_cast<const TT*>(A), lda, reinterpret_cast<const TT*>(B), ldb, b_expert_stride,    \
@@ -322,12 +307,7 @@ extern "C" int fx_grouped_gemm_wgrad(const void* A, int64_t lda, const void* B, 
     {                                                                                                     \
         auto kern = grouped_wgrad_kernel<TT, TG, BM, BN, 2, 4>;                                           \
         constexpr size_t lds = gemm2_lds_bytes<TT, BM, BN, 2, 4>();                                       \
-        static bool attr_set = false;                                                                     \
-        if (!attr_set) {                                                                                  \
-            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                \
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);              \
-            attr_set = true;                                                                              \
-        }                                                                                                 \
+        FX_ENSURE_DYNAMIC_LDS(kern, lds);                                                                 \
         kern<<<grid, 2 * 4 * 64, lds, stream>>>(reinterpret_cast<const TT*>(A), lda,                      \
                                                 reinterpret_cast<const TT*>(B), ldb, reinterpret_cast<TG*>(G), \
                                                 ldg, g_expert_stride, w.offsets, M, N, alpha, beta, tiles_n, tiles_m * tiles_n); \
