@@ -80,14 +80,20 @@ extern "C" int fx_adamw_stream_chunk(void* p_host, const void* g_host, void* m_h
         FX_FAIL("fx_adamw_stream_chunk: workspace too small (%zu < %zu bytes)", ws_bytes, L.stride * (size_t)n_slots);
 
     const size_t psz = elem_size(p_dt), gsz = elem_size(g_dt), ssz = elem_size(state_dt);
-    hipEvent_t in_done[16], k_done[16], out_done[16];
+    hipEvent_t in_done[16] = {}, k_done[16] = {}, out_done[16] = {};
     int made = 0, rc = 0;
     for (; made < n_slots; ++made) {
         if (hipEventCreateWithFlags(&in_done[made], hipEventDisableTiming) != hipSuccess ||
             hipEventCreateWithFlags(&k_done[made], hipEventDisableTiming) != hipSuccess ||
             hipEventCreateWithFlags(&out_done[made], hipEventDisableTiming) != hipSuccess) {
             fprintf(stderr, "flexhip: fx_adamw_stream_chunk: event creation failed\n");
-            return -1;  // events of earlier slots leak only on this failure path
+            (void)hipGetLastError();
+            for (int s = 0; s <= made; ++s) {      // the failing slot may hold one or two live events
+                if (in_done[s]) (void)hipEventDestroy(in_done[s]);
+                if (k_done[s]) (void)hipEventDestroy(k_done[s]);
+                if (out_done[s]) (void)hipEventDestroy(out_done[s]);
+            }
+            return -1;
         }
     }
     {
