@@ -3,7 +3,7 @@
 // out = act(x1) * x3, x1 = gate, x3 = up/value.  Math follows the reference
 // Triton kernels: flextrain/ops/_kernels/swiglu.py:9-96 and
 // flextrain/ops/_kernels/gelu_tanh_gated.py:55-140.  Pure streaming kernels:
-// every lane moves 16 bytes per tensor per access, two packs per lane.
+// every lane moves 16 bytes per tensor per access, one pack per lane.
 #include "common.h"
 #include "flexhip.h"
 
@@ -36,18 +36,24 @@ FX_DEV void glu_bwd_elem(float x1, float x3, float dout, float& dx1, float& dx3,
     }
 }
 
-constexpr int GLU_THREADS = 256;
-constexpr int GLU_UNROLL = 2;  // packs of 8 per lane
+// Workgroup size and packs of 8 elements per lane, from a sweep at the [8192, 14336] bf16 shape:
+// one pack per lane beats two or four; the forward kernel (two input streams) is fastest with
+// 512 lanes (6.06 TB/s against 5.68 at 256 x 2), the backward kernel (three input, two or three
+// output streams) with 1024 (6.20 TB/s against 5.86).
+constexpr int GLU_FWD_THREADS = 512;
+constexpr int GLU_BWD_THREADS = 1024;
+constexpr int GLU_THREADS = 512;  // SiLU backward
+constexpr int GLU_UNROLL = 1;
 
 template <typename T, typename TO, int ACT, bool NT>
-__global__ __launch_bounds__(GLU_THREADS) void glu_fwd_kernel(
+__global__ __launch_bounds__(GLU_FWD_THREADS) void glu_fwd_kernel(
     const T* __restrict__ X1, const T* __restrict__ X3, TO* __restrict__ OUT, int64_t n) {
-    const int64_t base = ((int64_t)blockIdx.x * GLU_UNROLL) * GLU_THREADS * 8;
+    const int64_t base = ((int64_t)blockIdx.x * GLU_UNROLL) * GLU_FWD_THREADS * 8;
     float a[GLU_UNROLL][8], b[GLU_UNROLL][8];
     bool full[GLU_UNROLL];
 #pragma unroll
     for (int u = 0; u < GLU_UNROLL; ++u) {
-        const int64_t off = base + ((int64_t)u * GLU_THREADS + threadIdx.x) * 8;
+        const int64_t off = base + ((int64_t)u * GLU_FWD_THREADS + threadIdx.x) * 8;
         full[u] = off + 8 <= n;
         if (full[u]) {
             load_f32<T, 8, NT>(X1 + off, a[u]);
@@ -56,7 +62,7 @@ __global__ __launch_bounds__(GLU_THREADS) void glu_fwd_kernel(
     }
 #pragma unroll
     for (int u = 0; u < GLU_UNROLL; ++u) {
-        const int64_t off = base + ((int64_t)u * GLU_THREADS + threadIdx.x) * 8;
+        const int64_t off = base + ((int64_t)u * GLU_FWD_THREADS + threadIdx.x) * 8;
         if (full[u]) {
             float o[8];
 #pragma unroll
@@ -70,15 +76,15 @@ __global__ __launch_bounds__(GLU_THREADS) void glu_fwd_kernel(
 }
 
 template <typename T, int ACT, bool STORE_ACT, bool NT>
-__global__ __launch_bounds__(GLU_THREADS) void glu_bwd_kernel(
+__global__ __launch_bounds__(GLU_BWD_THREADS) void glu_bwd_kernel(
     const T* __restrict__ X1, const T* __restrict__ X3, const T* __restrict__ DOUT,
     T* __restrict__ DX1, T* __restrict__ DX3, T* __restrict__ ACTOUT, int64_t n) {
-    const int64_t base = ((int64_t)blockIdx.x * GLU_UNROLL) * GLU_THREADS * 8;
+    const int64_t base = ((int64_t)blockIdx.x * GLU_UNROLL) * GLU_BWD_THREADS * 8;
     float a[GLU_UNROLL][8], b[GLU_UNROLL][8], d[GLU_UNROLL][8];
     bool full[GLU_UNROLL];
 #pragma unroll
     for (int u = 0; u < GLU_UNROLL; ++u) {
-        const int64_t off = base + ((int64_t)u * GLU_THREADS + threadIdx.x) * 8;
+        const int64_t off = base + ((int64_t)u * GLU_BWD_THREADS + threadIdx.x) * 8;
         full[u] = off + 8 <= n;
         if (full[u]) {
             load_f32<T, 8, NT>(X1 + off, a[u]);
@@ -88,7 +94,7 @@ __global__ __launch_bounds__(GLU_THREADS) void glu_bwd_kernel(
     }
 #pragma unroll
     for (int u = 0; u < GLU_UNROLL; ++u) {
-        const int64_t off = base + ((int64_t)u * GLU_THREADS + threadIdx.x) * 8;
+        const int64_t off = base + ((int64_t)u * GLU_BWD_THREADS + threadIdx.x) * 8;
         if (full[u]) {
             float g1[8], g3[8], ac[8];
 #pragma unroll
@@ -164,12 +170,12 @@ static void launch_glu_fwd(const void* x1, const void* x3, void* out, int64_t n,
     const T* b = reinterpret_cast<const T*>(x3);
     TO* o = reinterpret_cast<TO*>(out);
     if (aligned16(x1) && aligned16(x3) && aligned16(out)) {
-        const int64_t per_block = (int64_t)GLU_UNROLL * GLU_THREADS * 8;
+        const int64_t per_block = (int64_t)GLU_UNROLL * GLU_FWD_THREADS * 8;
         const unsigned grid = (unsigned)((n + per_block - 1) / per_block);
         if ((size_t)n * (2 * sizeof(T) + sizeof(TO)) >= kStreamingBytes)
-            glu_fwd_kernel<T, TO, ACT, true><<<grid, GLU_THREADS, 0, s>>>(a, b, o, n);
+            glu_fwd_kernel<T, TO, ACT, true><<<grid, GLU_FWD_THREADS, 0, s>>>(a, b, o, n);
         else
-            glu_fwd_kernel<T, TO, ACT, false><<<grid, GLU_THREADS, 0, s>>>(a, b, o, n);
+            glu_fwd_kernel<T, TO, ACT, false><<<grid, GLU_FWD_THREADS, 0, s>>>(a, b, o, n);
     } else {
         glu_fwd_scalar_kernel<T, TO, ACT><<<(unsigned)((n + 255) / 256), 256, 0, s>>>(a, b, o, n);
     }
@@ -186,13 +192,13 @@ static void launch_glu_bwd(const void* x1, const void* x3, const void* dout, voi
     T* ac = reinterpret_cast<T*>(act);
     if (aligned16(x1) && aligned16(x3) && aligned16(dout) && aligned16(dx1) && aligned16(dx3) &&
         (act == nullptr || aligned16(act))) {
-        const int64_t per_block = (int64_t)GLU_UNROLL * GLU_THREADS * 8;
+        const int64_t per_block = (int64_t)GLU_UNROLL * GLU_BWD_THREADS * 8;
         const unsigned grid = (unsigned)((n + per_block - 1) / per_block);
         const bool nt = (size_t)n * 5 * sizeof(T) >= kStreamingBytes;
-        if (act && nt) glu_bwd_kernel<T, ACT, true, true><<<grid, GLU_THREADS, 0, s>>>(a, b, d, g1, g3, ac, n);
-        else if (act) glu_bwd_kernel<T, ACT, true, false><<<grid, GLU_THREADS, 0, s>>>(a, b, d, g1, g3, ac, n);
-        else if (nt) glu_bwd_kernel<T, ACT, false, true><<<grid, GLU_THREADS, 0, s>>>(a, b, d, g1, g3, ac, n);
-        else glu_bwd_kernel<T, ACT, false, false><<<grid, GLU_THREADS, 0, s>>>(a, b, d, g1, g3, ac, n);
+        if (act && nt) glu_bwd_kernel<T, ACT, true, true><<<grid, GLU_BWD_THREADS, 0, s>>>(a, b, d, g1, g3, ac, n);
+        else if (act) glu_bwd_kernel<T, ACT, true, false><<<grid, GLU_BWD_THREADS, 0, s>>>(a, b, d, g1, g3, ac, n);
+        else if (nt) glu_bwd_kernel<T, ACT, false, true><<<grid, GLU_BWD_THREADS, 0, s>>>(a, b, d, g1, g3, ac, n);
+        else glu_bwd_kernel<T, ACT, false, false><<<grid, GLU_BWD_THREADS, 0, s>>>(a, b, d, g1, g3, ac, n);
     } else {
         glu_bwd_scalar_kernel<T, ACT><<<(unsigned)((n + 255) / 256), 256, 0, s>>>(a, b, d, g1, g3, ac, n);
     }
