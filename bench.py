@@ -36,7 +36,7 @@ BF16_PEAK_TFLOPS = 2500.0    # MI355X dense bf16 MFMA, published
 # HBM bytes per launch of the SwiGLU backward kernel at the benchmark shape, from the FETCH_SIZE and
 # WRITE_SIZE hardware counters scaled by what they read for a plain copy of known size
 # (profiles/glu_bwd_hbm_traffic_pmc.txt holds the counter values and the commands).
-GLU_BWD_MEASURED_TRAFFIC_BYTES = 1_174_223_936
+GLU_BWD_MEASURED_TRAFFIC_BYTES = 1_174_285_231
 
 METRIC = "per-op HBM GB/s (% of 8 TB/s) + lm_head/MoE GEMM TFLOPS (% bf16 MFMA peak)"
 
