@@ -308,6 +308,14 @@ def run_lm_head(torch, dev, stream, rn):
     rows.append(_op_entry("c3.dW gemm [128256,1024]x[1024,4096] (+= fp32)", 2 * chunk * d * V, "TFLOP/s", ms))
     ms = _time_launches(torch, stream, [lambda: disp.matmul_fast(sp, logits, w, D=dxh)], warmup=2, reps=10)
     rows.append(_op_entry("c3.dX gemm [1024,128256]x[128256,4096]", 2 * chunk * d * V, "TFLOP/s", ms))
+    # For comparison only (not a product path): the vendor BLAS, which the reference's cuBLASLt
+    # dispatcher would map to on this hardware, on the same operands in the same run.
+    with torch.cuda.stream(stream):
+        ms = _time_launches(torch, stream, [lambda: torch.matmul(h, w.t(), out=logits)], warmup=2, reps=10)
+        rows.append(_op_entry("c3.logits gemm, vendor BLAS through torch.matmul (comparison)", 2 * chunk * d * V, "TFLOP/s", ms))
+        logits.normal_()
+        ms = _time_launches(torch, stream, [lambda: torch.matmul(logits, w, out=dxh)], warmup=2, reps=10)
+        rows.append(_op_entry("c3.dX gemm, vendor BLAS through torch.matmul (comparison)", 2 * chunk * d * V, "TFLOP/s", ms))
     from flextrain_amd import ops
     lab = labels[:chunk].contiguous()
     loss = torch.empty(chunk, dtype=torch.float32, device=dev)
@@ -425,7 +433,21 @@ def run_ffn_dense(torch, dev, stream, rn):
     unit = 2 * T * d * F
     ms_f = _time_launches(torch, stream, [fwd], warmup=2, reps=5)
     ms_b = _time_launches(torch, stream, [bwd], warmup=2, reps=5)
-    return [_op_entry("ffn.dense block fwd (3 GEMMs + SwiGLU, residual in the down-projection epilogue)", 3 * unit, "TFLOP/s", ms_f),
+    # single GEMMs of the block, and the vendor BLAS on the same operands for comparison
+    from flextrain_amd import ops
+    sp = stream.cuda_stream
+    x1 = slot.x1
+    extra_rows = []
+    ms = _time_launches(torch, stream, [lambda: ops.dispatcher.matmul_fast(sp, h, W["w_1"], D=x1)], warmup=2, reps=10)
+    extra_rows.append(_op_entry("ffn.gate gemm [8192,4096]x[4096,14336] (weights (d,F) as the reference stores them)", unit, "TFLOP/s", ms))
+    ms = _time_launches(torch, stream, [lambda: ops.dispatcher.matmul_fast(sp, act_buf, W["w_2"], D=out)], warmup=2, reps=10)
+    extra_rows.append(_op_entry("ffn.down gemm [8192,14336]x[14336,4096]", unit, "TFLOP/s", ms))
+    with torch.cuda.stream(stream):
+        ms = _time_launches(torch, stream, [lambda: torch.matmul(h, W["w_1"], out=x1)], warmup=2, reps=10)
+        extra_rows.append(_op_entry("ffn.gate gemm, vendor BLAS through torch.matmul (comparison)", unit, "TFLOP/s", ms))
+        ms = _time_launches(torch, stream, [lambda: torch.matmul(act_buf, W["w_2"], out=out)], warmup=2, reps=10)
+        extra_rows.append(_op_entry("ffn.down gemm, vendor BLAS through torch.matmul (comparison)", unit, "TFLOP/s", ms))
+    return extra_rows + [_op_entry("ffn.dense block fwd (3 GEMMs + SwiGLU, residual in the down-projection epilogue)", 3 * unit, "TFLOP/s", ms_f),
             _op_entry("ffn.dense block bwd (6 GEMMs + SwiGLU bwd)", 6 * unit, "TFLOP/s", ms_b),
             _op_entry("ffn.dense block fwd+bwd", 9 * unit, "TFLOP/s", ms_f + ms_b)]
 
