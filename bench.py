@@ -539,6 +539,9 @@ def main():
 
     import torch
 
+    import __graft_entry__
+    __graft_entry__.ensure_built()   # uses the library that is built; builds only when there is none
+
     from flextrain_amd import ops
     from flextrain_amd._lib import lib
 

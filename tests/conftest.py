@@ -13,6 +13,16 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 
 
+def pytest_sessionstart(session):
+    """The tests load the library that is built; only when none is there do they build it."""
+    from flextrain_amd._lib import LIB_PATH
+
+    if not os.path.exists(LIB_PATH):
+        import __graft_entry__
+
+        __graft_entry__.build()
+
+
 @pytest.fixture(scope="session")
 def dev():
     if not torch.cuda.is_available():
