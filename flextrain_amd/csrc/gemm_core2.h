@@ -220,6 +220,16 @@ FX_DEV void mma_step(const T* As, const T* Bs, int row_a0, int row_b0, int lane,
 // one K-step can run after the workgroup barrier while the first fragments of the next K-step are
 // being read.  Without that, every K-step starts with the matrix pipe idle for the LDS latency of
 // eight waves' first reads.
+// Compile-time index and loop: f(IntC<I>()) for I in [FROM, TO).
+template <int M> struct IntC { static constexpr int value = M; };
+template <int FROM, int TO, typename F>
+FX_DEV void static_for(F&& f) {
+    if constexpr (FROM < TO) {
+        f(IntC<FROM>());
+        static_for<FROM + 1, TO>(f);
+    }
+}
+
 // Swizzle of a K-contiguous tile whose rows hold BK k-values: 8 chunks per row (BK = 64) or 4 (BK = 32).
 template <int BK> FX_DEV int swz_k(int r) { return BK == 64 ? swz(r) : ((r >> 2) & 3); }
 
@@ -269,9 +279,12 @@ struct MmaPipe {
     }
     // MFMAs of the sub-step whose fragments sit in `cur`; with FETCH, the fragments of sub-step
     // ks_f of tiles (As_f, Bs_f) are read into `nxt`, one read after each of the first MFMAs.
-    template <bool FETCH, int M = 0>
+    // `after(IntC<M>)` runs in the shadow of MFMA M as well (the K loop hangs its global loads there).
+    struct Nothing { template <typename I> FX_DEV void operator()(I) const {} };
+
+    template <bool FETCH, int M = 0, typename After = Nothing>
     static FX_DEV void sub(f32x16_t (&acc)[TM][TN], const Slot& cur, Slot& nxt, const T* As_f, const T* Bs_f, int ks_f,
-                           int row_a0, int row_b0, int lane) {
+                           int row_a0, int row_b0, int lane, After&& after = After()) {
         if constexpr (M < MFMAS) {
             constexpr int i = M / TN, j = M % TN;
             __builtin_amdgcn_sched_barrier(0);
@@ -280,10 +293,57 @@ struct MmaPipe {
                 __builtin_amdgcn_sched_barrier(0);
                 fetch_one<M>(nxt, As_f, Bs_f, ks_f, row_a0, row_b0, lane);
             }
-            sub<FETCH, M + 1>(acc, cur, nxt, As_f, Bs_f, ks_f, row_a0, row_b0, lane);
+            __builtin_amdgcn_sched_barrier(0);
+            after(IntC<M>());
+            sub<FETCH, M + 1>(acc, cur, nxt, As_f, Bs_f, ks_f, row_a0, row_b0, lane, after);
         } else {
             __builtin_amdgcn_sched_barrier(0);
         }
+    }
+};
+
+// One operand tile's global -> LDS loads as separately issuable instructions: the per-lane source
+// pointers are worked out once and advanced by one K-step with every issue.
+template <typename T, int ROWS, int NW, bool MN, bool DUAL>
+struct TileLoader {
+    static constexpr int NI = ROWS / 8 / NW;    // 1 KB instructions per wave: ROWS x 128 bytes in all
+    static_assert(ROWS % (8 * NW) == 0, "tile rows must split evenly over the waves");
+    const T* src[NI];
+    int64_t step;
+
+    FX_DEV void init(const OperandView<T>& op, int wave, int lane) {
+        if (!MN) {
+            const int rr = lane >> 3, pos = lane & 7;
+#pragma unroll
+            for (int j = 0; j < NI; ++j) {
+                const int r = (j * NW + wave) * 8 + rr;
+                const bool second = DUAL && r >= op.half;
+                int g = op.origin + (second ? r - op.half : r);
+                g = g < op.ext ? g : op.ext - 1;
+                src[j] = (second ? op.base2 : op.base) + (int64_t)g * op.ld + (pos ^ swz(r)) * 8;
+            }
+            step = GEMM_BK;
+        } else {
+            constexpr int CPR = ROWS / 8, KPI = 64 / CPR;
+            static_assert(ROWS == 64 || ROWS == 128 || ROWS == 256, "unsupported tile rows");
+            const int kin = lane / CPR, pos = lane % CPR;
+#pragma unroll
+            for (int j = 0; j < NI; ++j) {
+                const int k = (j * NW + wave) * KPI + kin;
+                const int c = pos ^ (swz_tr(k) % CPR);
+                const bool second = DUAL && c * 8 >= op.half;
+                int g = op.origin + (second ? c * 8 - op.half : c * 8);
+                g = g + 8 <= op.ext ? g : op.ext - 8;
+                src[j] = (second ? op.base2 : op.base) + (int64_t)k * op.ld + g;
+            }
+            step = (int64_t)GEMM_BK * op.ld;
+        }
+    }
+    // instruction J of the next K-step not yet issued for J
+    template <int J>
+    FX_DEV void issue(T* lds, int wave) {
+        load_to_lds16(src[J], lds + (J * NW + wave) * 512);
+        src[J] += step;
     }
 };
 
@@ -407,21 +467,33 @@ FX_DEV void gemm_mainloop2(const OperandView<T>& A, const OperandView<T>& B, int
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
     const int nfull = K / GEMM_BK;  // K-steps that need no zero fill
-    auto issue = [&](int kt, T* buf) {
-        if (!A_MN) tile_load_direct<T, BM, NW>(A, kt * GEMM_BK, buf, wave, lane);
-        else tile_load_direct_tr<T, BM, NW>(A, kt * GEMM_BK, buf, wave, lane);
-        if (!B_MN) tile_load_direct<T, BN, NW, B_DUAL>(B, kt * GEMM_BK, buf + BM * GEMM_BK, wave, lane);
-        else tile_load_direct_tr<T, BN, NW, B_DUAL>(B, kt * GEMM_BK, buf + BM * GEMM_BK, wave, lane);
-    };
     static_assert(GEMM_BK == 64, "the pipeline below is written out for four sub-steps per K-step");
     if (nfull > 0) {
         typedef MmaPipe<T, BM, BN, WM, WN, A_MN, B_MN> Pipe;
+        typedef TileLoader<T, BM, NW, A_MN, false> LoadA;
+        typedef TileLoader<T, BN, NW, B_MN, B_DUAL> LoadB;
+        constexpr int LD = LoadA::NI + LoadB::NI;            // load instructions per wave and K-step
+        constexpr int PER = (LD + Pipe::MFMAS - 1) / Pipe::MFMAS;
+        // Measured: spreading the loads over the post-barrier MFMAs gains 2-3 % when both operands are
+        // K-contiguous and loses 7-30 % when one is read transposed (their loads then land too late).
+        constexpr bool HANG_LOADS = !A_MN && !B_MN;
+        LoadA la;
+        LoadB lb;
+        la.init(A, wave, lane);
+        lb.init(B, wave, lane);
+        // instruction IDX of the next K-step into the stage at `buf` (K-steps are issued in order)
+        auto issue_one = [&](auto idx, T* buf) {
+            constexpr int IDX = decltype(idx)::value;
+            if constexpr (IDX < LoadA::NI) la.template issue<IDX>(buf, wave);
+            else if constexpr (IDX < LD) lb.template issue<IDX - LoadA::NI>(buf + BM * GEMM_BK, wave);
+        };
+        auto issue = [&](T* buf) { static_for<0, LD>([&](auto idx) { issue_one(idx, buf); }); };
         typename Pipe::Slot f0, f1;
         const int ra = wm * WM, rb = wn * WN;
-        issue(0, smem);
+        issue(smem);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        if (nfull > 1) issue(1, smem + BUF);
+        if (nfull > 1) issue(smem + BUF);
         Pipe::fetch_all(f0, smem, smem + BM * GEMM_BK, 0, ra, rb, lane);
         for (int kt = 0; kt + 1 < nfull; ++kt) {
             T* cur = smem + (kt & 1) * BUF;
@@ -432,11 +504,20 @@ FX_DEV void gemm_mainloop2(const OperandView<T>& A, const OperandView<T>& B, int
             Pipe::template sub<true>(acc, f0, f1, cur, curb, 3, ra, rb, lane);
             // Every read of `cur` has been issued.  Once they and this wave's loads of step kt+1 have
             // landed, the barrier makes `nxt` readable and `cur` writable for everyone; the MFMAs of
-            // the last sub-step then run while the first fragments of step kt+1 are read.
+            // the last sub-step then run while the first fragments of step kt+1 are read and the
+            // loads of step kt+2 are issued into `cur` (PER of them after each MFMA, or all first).
             asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
             __syncthreads();
-            if (kt + 2 < nfull) issue(kt + 2, cur);
-            Pipe::template sub<true>(acc, f1, f0, nxt, nxt + BM * GEMM_BK, 0, ra, rb, lane);
+            const bool more = kt + 2 < nfull;
+            if constexpr (HANG_LOADS) {
+                Pipe::template sub<true>(acc, f1, f0, nxt, nxt + BM * GEMM_BK, 0, ra, rb, lane, [&](auto m) {
+                    constexpr int M = decltype(m)::value;
+                    if (more) static_for<M * PER, (M + 1) * PER>([&](auto idx) { issue_one(idx, cur); });
+                });
+            } else {
+                if (more) issue(cur);
+                Pipe::template sub<true>(acc, f1, f0, nxt, nxt + BM * GEMM_BK, 0, ra, rb, lane);
+            }
         }
         {   // last full K-step: nothing follows it in these buffers
             T* cur = smem + ((nfull - 1) & 1) * BUF;
