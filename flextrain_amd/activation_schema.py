@@ -199,32 +199,25 @@ def _match_to(src: torch.Tensor, dst: torch.Tensor) -> torch.Tensor:
 
 
 def _as_rows(t: torch.Tensor):
-    """(rows, row_bytes, pitch_bytes) of a tensor that is contiguous except for one outer stride,
-    or None when it has no such form."""
+    """``(rows, row_bytes, pitch_bytes)`` of a tensor that is ``rows`` equal contiguous pieces a
+    constant pitch apart (a contiguous tensor is one piece), or ``None`` when it has no such form.
+    A view narrowed along one axis of a contiguous tensor always has it."""
     es = t.element_size()
     if t.numel() == 0:
         return 0, 0, 0
     if t.is_contiguous():
         return 1, t.numel() * es, t.numel() * es
-    # find the split: dims [k:] contiguous among themselves, dims [:k] collapse to `rows` with one pitch
-    for k in range(1, t.dim()):
-        inner = t.shape[k:]
-        inner_numel = 1
-        for s in inner:
-            inner_numel *= s
-        expect = 1
-        ok = True
+    for k in range(1, t.dim()):            # dims [k:] form the piece, dims [:k] count the pieces
+        inner_numel, expect, ok = 1, 1, True
         for d in range(t.dim() - 1, k - 1, -1):
             if t.shape[d] != 1 and t.stride(d) != expect:
                 ok = False
                 break
             expect *= t.shape[d]
+            inner_numel *= t.shape[d]
         if not ok:
             continue
-        # outer dims must be collapsible with pitch = stride(k-1)
-        pitch = t.stride(k - 1)
-        rows = 1
-        expect = pitch
+        pitch, rows, expect = t.stride(k - 1), 1, t.stride(k - 1)
         for d in range(k - 1, -1, -1):
             if t.shape[d] != 1 and t.stride(d) != expect:
                 ok = False
@@ -236,44 +229,50 @@ def _as_rows(t: torch.Tensor):
     return None
 
 
+def _copy_desc(dst: torch.Tensor, src: torch.Tensor):
+    """``(rows, row_bytes, dst_pitch, src_pitch)`` for one linear or 2-D copy, or ``None``."""
+    rd, rs = _as_rows(dst), _as_rows(src)
+    if rd is None or rs is None:
+        return None
+    if rd[0] == 1 and rs[0] == 1:
+        return 1, rd[1], rd[1], rs[1]
+    if rd[0] == 1:                          # contiguous destination, pitched source
+        return rs[0], rs[1], rs[1], rs[2]
+    if rs[0] == 1:                          # pitched destination, contiguous source
+        return rd[0], rd[1], rd[2], rd[1]
+    if rd[:2] == rs[:2]:                    # both pitched, same pieces
+        return rd[0], rd[1], rd[2], rs[2]
+    return None
+
+
+_DIRECTION = {(False, True): 0, (True, False): 1, (True, True): 2}    # (dst on device, src on device)
+
+
 def copy_fields(pairs: Sequence[tuple], *, non_blocking: bool = True) -> None:
     """Copy ``src -> dst`` for every ``(dst, src)`` pair with one library call per direction, on the
     current stream.  Host tensors must be pinned for the copies to overlap with compute."""
     by_dir = {}
-    fallback = []
+    strided = []
     for dst, src in pairs:
         if dst.shape != src.shape or dst.dtype != src.dtype:
             raise ValueError(f"copy_fields: {tuple(src.shape)} {src.dtype} -> {tuple(dst.shape)} {dst.dtype}")
         if dst.numel() == 0:
             continue
-        direction = {(False, True): 0, (True, False): 1, (True, True): 2}.get((dst.is_cuda, src.is_cuda))
-        rd, rs = _as_rows(dst), _as_rows(src)
-        if direction is None or rd is None or rs is None:
-            fallback.append((dst, src))
+        direction = _DIRECTION.get((dst.is_cuda, src.is_cuda))
+        desc = _copy_desc(dst, src) if direction is not None else None
+        if desc is None:
+            strided.append((dst, src))
             continue
-        if rd[0] == 1 and rs[0] == 1:
-            rows, row_bytes, dp, sp = 1, rd[1], rd[1], rs[1]
-        elif rd[0] == 1 or rs[0] == 1 or rd[:2] != rs[:2]:
-            # one side contiguous, the other pitched: describe both with the pitched side's rows
-            pitched = rs if rd[0] == 1 else rd
-            if rd[0] != 1 and rs[0] != 1:
-                fallback.append((dst, src))
-                continue
-            rows, row_bytes = pitched[0], pitched[1]
-            dp = rd[2] if rd[0] != 1 else row_bytes
-            sp = rs[2] if rs[0] != 1 else row_bytes
-        else:
-            rows, row_bytes, dp, sp = rd[0], rd[1], rd[2], rs[2]
-        by_dir.setdefault((direction, dst.device if dst.is_cuda else src.device), []).append(
-            (dst.data_ptr(), src.data_ptr(), rows, row_bytes, dp, sp))
+        device = dst.device if dst.is_cuda else src.device
+        by_dir.setdefault((direction, device), []).append((dst.data_ptr(), src.data_ptr()) + desc)
     for (direction, device), items in by_dir.items():
         n = len(items)
         P, I = ctypes.c_void_p * n, ctypes.c_int64 * n
-        rc = lib().fx_copy_fields(n, P(*[i[0] for i in items]), P(*[i[1] for i in items]), I(*[i[2] for i in items]),
-                                  I(*[i[3] for i in items]), I(*[i[4] for i in items]), I(*[i[5] for i in items]),
+        cols = list(zip(*items))
+        rc = lib().fx_copy_fields(n, P(*cols[0]), P(*cols[1]), I(*cols[2]), I(*cols[3]), I(*cols[4]), I(*cols[5]),
                                   direction, stream_ptr(device))
         check(rc, "fx_copy_fields")
-    for dst, src in fallback:          # exotic strides: the framework's strided copy
+    for dst, src in strided:               # no single 2-D form (or host to host): the framework's strided copy
         dst.copy_(src, non_blocking=non_blocking)
     if not non_blocking:
         torch.cuda.current_stream().synchronize()

@@ -130,3 +130,17 @@ def test_rows_and_pitch_of_narrowed_views():
     assert _as_rows(u[:, :2, :5]) is None                       # two different pitches: no single 2-D form
     assert _as_rows(torch.zeros(0, 4)) == (0, 0, 0)
     assert _as_rows(t.t()) is None
+
+
+def test_copy_descriptor_pairs():
+    from flextrain_amd.activation_schema import _copy_desc
+
+    full = torch.zeros(6, 10, dtype=bf)
+    home = torch.zeros(6, 7, dtype=bf)
+    assert _copy_desc(home, full[:, :7]) == (6, 14, 14, 20)          # contiguous home <- narrowed ring view
+    assert _copy_desc(full[:, :7], home) == (6, 14, 20, 14)          # and back
+    assert _copy_desc(home, home.clone()) == (1, 84, 84, 84)
+    other = torch.zeros(6, 12, dtype=bf)
+    assert _copy_desc(full[:, :7], other[:, :7]) == (6, 14, 20, 24)  # both pitched, same pieces
+    assert _copy_desc(home, full.t()[:7].t()) == (6, 14, 14, 20)
+    assert _copy_desc(home.t(), full[:, :7].t()) is None             # transposed views: no 2-D form
