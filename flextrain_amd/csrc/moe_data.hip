@@ -82,17 +82,29 @@ __global__ __launch_bounds__(256) void moe_gather_kernel(
 #pragma unroll
                 for (int j = 0; j < 8; ++j) acc[j] = 0.f;
             }
-            for (int k = 0; k < K; ++k) {
-                const int64_t row = load_index(IDX, idx64, t * K + k);
-                float v[8];
-                load_f32<T, 8>(Y + row * D + c, v);
-                if (W != nullptr) {
-                    const float w = (float)W[t * K + k];
+            // rows of up to 4 slots are all requested before the first is added (k ascending, as
+            // the reference sums): one exposed memory round trip per batch instead of one per slot
+            for (int k0 = 0; k0 < K; k0 += 4) {
+                float v[4][8], w[4];
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) acc[j] += v[j] * w;
-                } else {
+                for (int u = 0; u < 4; ++u) {
+                    if (k0 + u < K) {
+                        const int64_t row = load_index(IDX, idx64, t * K + k0 + u);
+                        load_f32<T, 8>(Y + row * D + c, v[u]);
+                        w[u] = W != nullptr ? (float)W[t * K + k0 + u] : 1.f;
+                    }
+                }
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) acc[j] += v[j];
+                for (int u = 0; u < 4; ++u) {
+                    if (k0 + u < K) {
+                        if (W != nullptr) {
+#pragma unroll
+                            for (int j = 0; j < 8; ++j) acc[j] += v[u][j] * w[u];
+                        } else {
+#pragma unroll
+                            for (int j = 0; j < 8; ++j) acc[j] += v[u][j];
+                        }
+                    }
                 }
             }
             store_f32<TO, 8>(OUT + t * D + c, acc);
