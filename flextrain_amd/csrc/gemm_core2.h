@@ -35,8 +35,17 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 
 // 16 bytes per lane, global -> LDS; lds_base is wave-uniform, lane l lands at lds_base + 16*l.
+// Written as inline assembly on purpose.  With the compiler's builtin for this load, its wait-count
+// pass knows that LDS writes are in flight and puts `s_waitcnt vmcnt(0)` in front of every
+// ds_read_b64_tr_b16 that follows (it cannot tell that the reads touch the other buffer), which
+// exposes the whole global-load latency in every K-step of the transposed-read forms.  The loops
+// here wait for these loads themselves (`s_waitcnt vmcnt(n)` before the barrier that publishes a
+// buffer), so nothing else may depend on the compiler knowing about them.
+//   - the low half of a generic pointer into LDS is the LDS address;
+//   - an SALU write of M0 needs one wait state before an LDS-DMA instruction reads it.
 FX_DEV void load_to_lds16(const void* gptr, void* lds_base) {
-    __builtin_amdgcn_global_load_lds((gbl_ptr_t)gptr, (lds_ptr_t)lds_base, 16, 0, 0);
+    const unsigned lds_addr = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)lds_base);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(gptr) : "memory", "m0");
 }
 
 // Direct copy of a ROWS x 64 K-contiguous tile.  One wave instruction covers 8 rows
