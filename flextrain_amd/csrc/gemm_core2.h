@@ -31,8 +31,6 @@ namespace fx {
 // Swizzle: chunk c of row r sits at position c ^ swz(r).
 FX_DEV int swz(int r) { return (r >> GEMM_SWZ_SHIFT) & 7; }
 
-typedef __attribute__((address_space(3))) void* lds_ptr_t;
-typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 
 // 16 bytes per lane, global -> LDS; lds_base is wave-uniform, lane l lands at lds_base + 16*l.
 // Written as inline assembly on purpose.  With the compiler's builtin for this load, its wait-count
@@ -48,46 +46,9 @@ FX_DEV void load_to_lds16(const void* gptr, void* lds_base) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(gptr) : "memory", "m0");
 }
 
-// Direct copy of a ROWS x 64 K-contiguous tile.  One wave instruction covers 8 rows
-// (8 lanes per row); instruction j of wave w covers rows (j*NW + w)*8 ...
-template <typename T, int ROWS, int NW, bool DUAL = false>
-FX_DEV void tile_load_direct(const OperandView<T>& op, int k0, T* lds, int wave, int lane) {
-    constexpr int NI = ROWS / 8 / NW;
-    static_assert(ROWS % (8 * NW) == 0, "tile rows must split evenly over the waves");
-    const int rr = lane >> 3, pos = lane & 7;
-#pragma unroll
-    for (int j = 0; j < NI; ++j) {
-        const int r = (j * NW + wave) * 8 + rr;
-        const bool second = DUAL && r >= op.half;
-        int g = op.origin + (second ? r - op.half : r);
-        g = g < op.ext ? g : op.ext - 1;
-        const int c = pos ^ swz(r);
-        load_to_lds16((second ? op.base2 : op.base) + (int64_t)g * op.ld + k0 + c * 8, lds + (j * NW + wave) * 8 * GEMM_BK);
-    }
-}
-
-// Direct copy of a 64(k) x ROWS M/N-contiguous tile: LDS row k holds ROWS elements, its 16-byte
-// chunk c at position c ^ ((k & 3) << 2).  One wave instruction covers 1024 / (2*ROWS) k-rows.
+// LDS layout of a 64(k) x ROWS M/N-contiguous tile: row k holds ROWS elements, its 16-byte chunk c
+// at position c ^ ((k & 3) << 2).
 FX_DEV int swz_tr(int k) { return (k & 3) << 2; }
-
-template <typename T, int ROWS, int NW, bool DUAL = false>
-FX_DEV void tile_load_direct_tr(const OperandView<T>& op, int k0, T* lds, int wave, int lane) {
-    constexpr int NI = ROWS / 8 / NW;           // instructions per wave: ROWS * 128 bytes in all
-    constexpr int CPR = ROWS / 8;               // 16-byte chunks per LDS row
-    constexpr int KPI = 64 / CPR;               // k-rows per instruction
-    static_assert(ROWS % (8 * NW) == 0 && (ROWS == 64 || ROWS == 128 || ROWS == 256), "unsupported tile rows");
-    const int kin = lane / CPR, pos = lane % CPR;
-#pragma unroll
-    for (int j = 0; j < NI; ++j) {
-        const int q = j * NW + wave;
-        const int k = q * KPI + kin;
-        const int c = pos ^ (swz_tr(k) % CPR);
-        const bool second = DUAL && c * 8 >= op.half;
-        int g = op.origin + (second ? c * 8 - op.half : c * 8);
-        g = g + 8 <= op.ext ? g : op.ext - 8;
-        load_to_lds16((second ? op.base2 : op.base) + (int64_t)(k0 + k) * op.ld + g, lds + q * 512);
-    }
-}
 
 // Register-staged tile (any operand form, zero-fills k >= K) for NT threads.
 template <int ROWS, int NT>
