@@ -526,7 +526,12 @@ FX_DEV void gemm_tile2(const OperandView<T>& A, const OperandView<T>& B, const T
 // Per 32-row band every wave stages its fp32 results in LDS; after a barrier each wave of a pair
 // finishes 16 of the band's rows: reads both stagings, rounds, applies the activation and stores
 // the three outputs as 16-byte accesses.  Needs K % 64 == 0, Nh % 8 == 0, 16-byte aligned rows.
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool B_MN, int ACT>
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_MN, bool B_MN, bool B_DUAL = false>
+FX_DEV void gemm_mainloop32(const OperandView<T>& A, const OperandView<T>& B, int K, T* smem,
+                            f32x16_t (&acc)[BM / WAVES_M / 32][BN / WAVES_N / 32]);
+
+// K32: the K loop with 32-wide steps over three stages (K % 32 == 0) instead of 64-wide over two.
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool B_MN, int ACT, bool K32 = false>
 FX_DEV void gemm_tile2_glu(const OperandView<T>& A, const OperandView<T>& B, T* P1, T* P2, int64_t ldp, T* ACTO,
                            int64_t ldact, int M, int Nh, int K, bool gate_first, T* smem) {
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
@@ -538,7 +543,8 @@ FX_DEV void gemm_tile2_glu(const OperandView<T>& A, const OperandView<T>& B, T* 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
     f32x16_t acc[TM][TN];
-    gemm_mainloop2<T, BM, BN, WAVES_M, WAVES_N, false, B_MN, true>(A, B, K, smem, acc);
+    if constexpr (K32) gemm_mainloop32<T, BM, BN, WAVES_M, WAVES_N, false, B_MN, true>(A, B, K, smem, acc);
+    else gemm_mainloop2<T, BM, BN, WAVES_M, WAVES_N, false, B_MN, true>(A, B, K, smem, acc);
 
     float* stage = reinterpret_cast<float*>(smem) + wave * 32 * PITCH;
     const bool second = wn >= HW;
@@ -593,7 +599,7 @@ FX_DEV void gemm_tile2_glu(const OperandView<T>& A, const OperandView<T>& B, T* 
 //     c ^ ((r >> 2) & 3) (16 consecutive rows of one chunk column hit 64 distinct banks); a wave
 //     instruction covers 16 rows.
 //   M/N-contiguous tile: as in the 64-wide form (row k holds the tile's m or n values), 32 rows.
-template <typename T, int ROWS, int NW>
+template <typename T, int ROWS, int NW, bool DUAL = false>
 FX_DEV void tile32_load_direct(const OperandView<T>& op, int k0, T* lds, int wave, int lane) {
     constexpr int NI = ROWS / 16 / NW;
     static_assert(ROWS % (16 * NW) == 0, "tile rows must split evenly over the waves");
@@ -601,14 +607,15 @@ FX_DEV void tile32_load_direct(const OperandView<T>& op, int k0, T* lds, int wav
 #pragma unroll
     for (int j = 0; j < NI; ++j) {
         const int r = (j * NW + wave) * 16 + rr;
-        int g = op.origin + r;
+        const bool second = DUAL && r >= op.half;
+        int g = op.origin + (second ? r - op.half : r);
         g = g < op.ext ? g : op.ext - 1;
         const int c = pos ^ swz_k<32>(r);
-        load_to_lds16(op.base + (int64_t)g * op.ld + k0 + c * 8, lds + (j * NW + wave) * 16 * 32);
+        load_to_lds16((second ? op.base2 : op.base) + (int64_t)g * op.ld + k0 + c * 8, lds + (j * NW + wave) * 16 * 32);
     }
 }
 
-template <typename T, int ROWS, int NW>
+template <typename T, int ROWS, int NW, bool DUAL = false>
 FX_DEV void tile32_load_direct_tr(const OperandView<T>& op, int k0, T* lds, int wave, int lane) {
     constexpr int CPR = ROWS / 8;               // 16-byte chunks per LDS row
     constexpr int KPI = 64 / CPR;               // k-rows per instruction
@@ -620,9 +627,10 @@ FX_DEV void tile32_load_direct_tr(const OperandView<T>& op, int k0, T* lds, int 
         const int q = j * NW + wave;
         const int k = q * KPI + kin;
         const int c = pos ^ (swz_tr(k) % CPR);
-        int g = op.origin + c * 8;
+        const bool second = DUAL && c * 8 >= op.half;
+        int g = op.origin + (second ? c * 8 - op.half : c * 8);
         g = g + 8 <= op.ext ? g : op.ext - 8;
-        load_to_lds16(op.base + (int64_t)(k0 + k) * op.ld + g, lds + q * 512);
+        load_to_lds16((second ? op.base2 : op.base) + (int64_t)(k0 + k) * op.ld + g, lds + q * 512);
     }
 }
 
@@ -635,7 +643,7 @@ constexpr size_t gemm32_lds_bytes() {
 
 // K loop with 32-wide steps over three rotating LDS stages; K must be a multiple of 32.
 // Leaves the accumulators in `acc` and ends with a barrier (the stages become epilogue staging).
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_MN, bool B_MN>
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_MN, bool B_MN, bool B_DUAL>
 FX_DEV void gemm_mainloop32(const OperandView<T>& A, const OperandView<T>& B, int K, T* smem,
                             f32x16_t (&acc)[BM / WAVES_M / 32][BN / WAVES_N / 32]) {
     constexpr int NW = WAVES_M * WAVES_N;
@@ -656,8 +664,8 @@ FX_DEV void gemm_mainloop32(const OperandView<T>& A, const OperandView<T>& B, in
     auto issue = [&](int kt, T* buf) {
         if (!A_MN) tile32_load_direct<T, BM, NW>(A, kt * 32, buf, wave, lane);
         else tile32_load_direct_tr<T, BM, NW>(A, kt * 32, buf, wave, lane);
-        if (!B_MN) tile32_load_direct<T, BN, NW>(B, kt * 32, buf + BM * 32, wave, lane);
-        else tile32_load_direct_tr<T, BN, NW>(B, kt * 32, buf + BM * 32, wave, lane);
+        if (!B_MN) tile32_load_direct<T, BN, NW, B_DUAL>(B, kt * 32, buf + BM * 32, wave, lane);
+        else tile32_load_direct_tr<T, BN, NW, B_DUAL>(B, kt * 32, buf + BM * 32, wave, lane);
     };
     if (n > 0) {
         typedef MmaPipe<T, BM, BN, WM, WN, A_MN, B_MN, 32> Pipe;

@@ -128,8 +128,8 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64, 2) void grouped_rows_kernel
 // Up projection of every expert with the SwiGLU in the epilogue: the expert's weight holds two
 // Nh-row (or Nh-column) halves b2_delta elements apart; P1 / P2 receive the two pre-activation
 // halves and ACTO the gated product (see gemm_tile2_glu).
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool B_MN>
-__global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void grouped_rows_glu_kernel(
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool B_MN, bool K32 = false>
+__global__ __launch_bounds__(WAVES_M * WAVES_N * 64, K32 ? 2 : 1) void grouped_rows_glu_kernel(
     const T* __restrict__ A, int64_t lda, const T* __restrict__ B, int64_t ldb, int64_t b_expert_stride,
     int64_t b2_delta, T* P1, T* P2, int64_t ldp, T* ACTO, int64_t ldact, const int32_t* __restrict__ NTILES,
     const int32_t* __restrict__ OFFSETS, const int32_t* __restrict__ TILES, int Nh, int K, int gate_first,
@@ -148,9 +148,9 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void grouped_rows_glu_kerne
     OperandView<T> a{A + row0 * lda, lda, rows, m0};
     const T* b1 = B + (int64_t)e * b_expert_stride;
     OperandView<T> b{b1, ldb, Nh, tn * (BN / 2), BN / 2, b1 + b2_delta};
-    gemm_tile2_glu<T, BM, BN, WAVES_M, WAVES_N, B_MN, ACT_SILU>(a, b, P1 + row0 * ldp, P2 + row0 * ldp, ldp,
-                                                                ACTO + row0 * ldact, ldact, rows, Nh, K,
-                                                                gate_first != 0, smem);
+    gemm_tile2_glu<T, BM, BN, WAVES_M, WAVES_N, B_MN, ACT_SILU, K32>(a, b, P1 + row0 * ldp, P2 + row0 * ldp, ldp,
+                                                                     ACTO + row0 * ldact, ldact, rows, Nh, K,
+                                                                     gate_first != 0, smem);
 }
 
 template <typename T, typename TG, int BM, int BN, int WAVES_M, int WAVES_N>
@@ -265,10 +265,11 @@ extern "C" int fx_grouped_gemm_rows_glu(const void* A, int64_t lda, const void* 
     grouped_plan_kernel<<<1, 256, 0, stream>>>(counts, E, BM, w.ntiles, w.offsets, w.tiles);
     FX_CHECK_LAUNCH("fx_grouped_gemm_rows_glu(plan)");
     const unsigned max_tiles = (unsigned)(total_rows / BM + E);
-#define FX_GLU(TT, BM_, BN_, WM_, WN_, BMN)                                                               \
+#define FX_GLU(TT, BM_, BN_, WM_, WN_, BMN, K32_)                                                         \
     {                                                                                                     \
-        auto kern = grouped_rows_glu_kernel<TT, BM_, BN_, WM_, WN_, BMN>;                                 \
-        constexpr size_t lds = gemm2_lds_bytes<TT, BM_, BN_, WM_, WN_>();                                 \
+        auto kern = grouped_rows_glu_kernel<TT, BM_, BN_, WM_, WN_, BMN, K32_>;                           \
+        constexpr size_t lds = K32_ ? gemm32_lds_bytes<TT, BM_, BN_, WM_, WN_>()                          \
+                                    : gemm2_lds_bytes<TT, BM_, BN_, WM_, WN_>();                          \
         FX_ENSURE_DYNAMIC_LDS(kern, lds);                                                                 \
         const int tiles_n = cdiv_i(Nh, BN_ / 2);                                                          \
         kern<<<dim3(max_tiles * (unsigned)tiles_n), WM_ * WN_ * 64, lds, stream>>>(                       \
@@ -276,9 +277,10 @@ extern "C" int fx_grouped_gemm_rows_glu(const void* A, int64_t lda, const void* 
             b2_delta, reinterpret_cast<TT*>(P1), reinterpret_cast<TT*>(P2), ldp, reinterpret_cast<TT*>(act), \
             ldact, w.ntiles, w.offsets, w.tiles, Nh, K, gate_first, tiles_n);                             \
     }
+    // 128-row tiles: 128 x 256 (128 columns of each half) with 32-wide K-steps, two workgroups per CU
 #define FX_GLU_T(TT)                                                                                      \
-    if (BM == 256) { if (trans_b) FX_GLU(TT, 256, 256, 2, 4, false) else FX_GLU(TT, 256, 256, 2, 4, true) } \
-    else { if (trans_b) FX_GLU(TT, 128, 128, 2, 2, false) else FX_GLU(TT, 128, 128, 2, 2, true) }
+    if (BM == 256) { if (trans_b) FX_GLU(TT, 256, 256, 2, 4, false, false) else FX_GLU(TT, 256, 256, 2, 4, true, false) } \
+    else { if (trans_b) FX_GLU(TT, 128, 256, 2, 2, false, true) else FX_GLU(TT, 128, 256, 2, 2, true, true) }
     if (dt == DT_BF16) { FX_GLU_T(bf16) } else { FX_GLU_T(f16) }
 #undef FX_GLU_T
 #undef FX_GLU
