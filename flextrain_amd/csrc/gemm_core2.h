@@ -25,11 +25,8 @@
 
 namespace fx {
 
-#ifndef GEMM_SWZ_SHIFT
-#define GEMM_SWZ_SHIFT 1
-#endif
 // Swizzle: chunk c of row r sits at position c ^ swz(r).
-FX_DEV int swz(int r) { return (r >> GEMM_SWZ_SHIFT) & 7; }
+FX_DEV int swz(int r) { return (r >> 1) & 7; }
 
 
 // 16 bytes per lane, global -> LDS; lds_base is wave-uniform, lane l lands at lds_base + 16*l.
