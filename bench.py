@@ -49,7 +49,7 @@ def _parse():
     ap.add_argument("--no-extra", action="store_true", help="skip the non-headline configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--only", default="", help="comma-separated subset of the non-headline configurations "
-                                               "(c1, c3, c4, c5, ffn, act, probe) to run, e.g. for a profiler pass")
+                                               "(c1, c3, c4, c5, ffn, attn, act, probe) to run, e.g. for a profiler pass")
     return ap.parse_args()
 
 
@@ -117,6 +117,8 @@ def run_extra(torch, ops, dev, stream, rn, only):
         rows += run_moe(torch, dev, stream, rn)
     if want("ffn"):
         rows += run_ffn_dense(torch, dev, stream, rn)
+    if want("attn"):
+        rows += run_attention_proj(torch, dev, stream, rn)
     if want("act"):
         rows += run_activation_slots(torch, dev)
     if want("probe"):
@@ -450,6 +452,46 @@ def run_ffn_dense(torch, dev, stream, rn):
     return extra_rows + [_op_entry("ffn.dense block fwd (3 GEMMs + SwiGLU, residual in the down-projection epilogue)", 3 * unit, "TFLOP/s", ms_f),
             _op_entry("ffn.dense block bwd (6 GEMMs + SwiGLU bwd)", 6 * unit, "TFLOP/s", ms_b),
             _op_entry("ffn.dense block fwd+bwd", 9 * unit, "TFLOP/s", ms_f + ms_b)]
+
+
+def run_attention_proj(torch, dev, stream, rn):
+    """Llama-3.1-8B-shaped attention block without its core (the projections around the RoPE kernel of
+    the headline workload): T = 8192 tokens, d = 4096, 32 query heads, 8 key/value heads of 128."""
+    import types
+
+    from flextrain_amd.attention_proj import GQAAttentionProjections, GQAProjectionConfig
+
+    T = 8192
+    cfg = GQAProjectionConfig(d_model=4096, n_heads=32, n_kv_heads=8, head_dim=128, rope_theta=500000.0)
+    bf = torch.bfloat16
+    x, resid, dy = rn(T, cfg.d_model).to(dev), rn(T, cfg.d_model).to(dev), rn(T, cfg.d_model).to(dev)
+    pos = torch.arange(T, dtype=torch.int32, device=dev).view(T, 1)
+    shapes = {"q": (cfg.d_model, cfg.attn_dim), "k": (cfg.d_model, cfg.kv_dim), "v": (cfg.d_model, cfg.kv_dim),
+              "o": (cfg.attn_dim, cfg.d_model)}
+    W = {"w_" + k: (torch.randn(*sh, device=dev) * 0.02).to(bf) for k, sh in shapes.items()}
+    G = {"g_" + k: torch.zeros(*sh, dtype=bf, device=dev) for k, sh in shapes.items()}
+    slot = types.SimpleNamespace(
+        xq=torch.empty(T, cfg.n_heads, cfg.head_dim, dtype=bf, device=dev), xk=torch.empty(T, cfg.n_kv_heads, cfg.head_dim, dtype=bf, device=dev),
+        xv=torch.empty(T, cfg.n_kv_heads, cfg.head_dim, dtype=bf, device=dev), attn_result=rn(T, cfg.n_heads, cfg.head_dim).to(dev),
+        xo=torch.empty(T, cfg.d_model, dtype=bf, device=dev), aux={})
+    dq, dk, dv = rn(T, cfg.n_heads, cfg.head_dim).to(dev), rn(T, cfg.n_kv_heads, cfg.head_dim).to(dev), rn(T, cfg.n_kv_heads, cfg.head_dim).to(dev)
+    blk = GQAAttentionProjections(cfg)
+
+    def fwd():
+        blk.fwd_qkv(x, pos, W, slot)
+        blk.fwd_o(resid, W, slot)
+
+    def bwd():
+        blk.bwd_o(dy, W, G, slot)
+        blk.bwd_qkv(dq, dk, dv, pos, W, G, slot)
+        blk.bwd_accumulate_qkv_grads(x, G, slot)
+
+    fl = blk.projection_flops(T)
+    ms_f = _time_launches(torch, stream, [fwd], warmup=2, reps=5)
+    ms_b = _time_launches(torch, stream, [bwd], warmup=2, reps=5)
+    return [_op_entry("attn.projections fwd (Q/K/V GEMMs + RoPE, O-projection with the residual in its epilogue)", fl, "TFLOP/s", ms_f),
+            _op_entry("attn.projections bwd (8 GEMMs + RoPE bwd)", 2 * fl, "TFLOP/s", ms_b),
+            _op_entry("attn.projections fwd+bwd", 3 * fl, "TFLOP/s", ms_f + ms_b)]
 
 
 def run_moe(torch, dev, stream, rn):

@@ -27,6 +27,13 @@ How each function is pinned (tests/test_oracle_*.py, all CPU-only):
                torch.autograd through rms_norm -> matmul -> cross-entropy.
   moe          stable sort / bincount / indexing identities, torch.autograd through
                the eager expert formula (tests/moe/test_moe_backend_parity.py:45-107).
+  ffn_dense    torch.autograd through the textbook gated-FFN formula in fp32 (both
+               activations), weight gradients accumulated onto given tensors.
+  attention_proj  torch.autograd through an independent fp32 formulation of the attention
+               block (projections with biases, F.rms_norm per head, RoPE as complex
+               multiplication, dense causal grouped-query attention as the core, output
+               projection plus residual): each half is fed autograd's own tensors at the
+               core's boundary and must return autograd's gradients.
   dp_solver    golden vectors from the compiled reference solver (oracle/_ref, built
                by oracle/Makefile from the reference's own C file), the README known
                answer, exhaustive enumeration of all option vectors on small problems.
