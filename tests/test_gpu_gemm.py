@@ -30,7 +30,8 @@ def _check(D, want, dtype):
 
 
 SHAPES = [(200, 1024, 2048), (500, 2048, 512), (37, 16, 4096), (16, 1024, 16), (256, 256, 64), (1024, 1536, 2048),
-          (513, 768, 2048), (128, 128, 8), (1, 8, 8), (3000, 4096, 1024)]
+          (513, 768, 2048), (128, 128, 8), (1, 8, 8), (3000, 4096, 1024),
+          (2040, 3200, 200)]   # the last one takes the 256 x 128 tile (one full round of workgroups), ragged in M and K
 
 
 @pytest.mark.parametrize("M,N,K", SHAPES)
