@@ -38,6 +38,25 @@ FX_DEV void stat_add(RowStat& s, float x, int i) {
     }
 }
 
+// Eight consecutive elements at once: one rescale of the running sum per pack instead of a
+// data-dependent branch per element (the sweep is otherwise bound by its exponentials).
+FX_DEV void stat_add_pack(RowStat& s, const float (&v)[8], int c0) {
+    float pm = v[0];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        if (v[j] > s.best) { s.best = v[j]; s.idx = c0 + j; }   // strict: the first maximum wins
+        pm = fmaxf(pm, v[j]);
+    }
+    if (pm > NEG_INF_F) {                 // a pack of -inf adds nothing (and -inf - -inf is NaN)
+        const float nm = fmaxf(s.m, pm);
+        float acc = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc += __expf(v[j] - nm);
+        s.l = s.l * __expf(s.m - nm) + acc;
+        s.m = nm;
+    }
+}
+
 FX_DEV void stat_merge(RowStat& a, float m, float l, float best, int idx) {
     if (best > a.best || (best == a.best && idx < a.idx)) { a.best = best; a.idx = idx; }
     const float nm = fmaxf(a.m, m);
@@ -72,7 +91,8 @@ FX_DEV RowStat row_sweep(const T* __restrict__ x, int V, float inv_temp, bool ve
             float v[8];
             load_f32<T, 8>(x + c, v);
 #pragma unroll
-            for (int j = 0; j < 8; ++j) stat_add(s, v[j] * inv_temp, c + j);
+            for (int j = 0; j < 8; ++j) v[j] *= inv_temp;
+            stat_add_pack(s, v, c);
         }
     } else {
         for (int c = threadIdx.x; c < V; c += SM_THREADS) stat_add(s, (float)x[c] * inv_temp, c);
