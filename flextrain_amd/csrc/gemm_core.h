@@ -39,10 +39,15 @@ struct OperandView {
     int64_t ld;
     int ext;
     int origin;
-    // Two-matrix tile (loaders instantiated with DUAL): tile rows >= half come from the matrix
-    // at `base2` (same ld and extent), at index origin + row - half.
+    // Two-matrix tile (loaders instantiated with DUAL): tile rows alternate between the two matrices
+    // in blocks of `half` (a power of two): rows [0, half) are indices origin + [0, half) of `base`,
+    // rows [half, 2 half) the same indices of `base2` (same ld and extent), rows [2 half, 3 half)
+    // indices origin + [half, 2 half) of `base` again, and so on.
     int half = 0;
     const T* base2 = nullptr;
+    // tile row -> which matrix, and the index offset from `origin`
+    __device__ __forceinline__ bool dual_second(int r) const { return (r & half) != 0; }
+    __device__ __forceinline__ int dual_index(int r) const { return ((r & ~(2 * half - 1)) >> 1) + (r & (half - 1)); }
 };
 
 FX_DEV u32x4_t ldg16(const void* p) { return *reinterpret_cast<const u32x4_t*>(p); }

@@ -284,8 +284,8 @@ struct TileLoader {
 #pragma unroll
             for (int j = 0; j < NI; ++j) {
                 const int r = (j * NW + wave) * 8 + rr;
-                const bool second = DUAL && r >= op.half;
-                int g = op.origin + (second ? r - op.half : r);
+                const bool second = DUAL && op.dual_second(r);
+                int g = op.origin + (DUAL ? op.dual_index(r) : r);
                 g = g < op.ext ? g : op.ext - 1;
                 src[j] = (second ? op.base2 : op.base) + (int64_t)g * op.ld + (pos ^ swz(r)) * 8;
             }
@@ -298,8 +298,8 @@ struct TileLoader {
             for (int j = 0; j < NI; ++j) {
                 const int k = (j * NW + wave) * KPI + kin;
                 const int c = pos ^ (swz_tr(k) % CPR);
-                const bool second = DUAL && c * 8 >= op.half;
-                int g = op.origin + (second ? c * 8 - op.half : c * 8);
+                const bool second = DUAL && op.dual_second(c * 8);
+                int g = op.origin + (DUAL ? op.dual_index(c * 8) : c * 8);
                 g = g + 8 <= op.ext ? g : op.ext - 8;
                 src[j] = (second ? op.base2 : op.base) + (int64_t)k * op.ld + g;
             }
@@ -517,73 +517,83 @@ FX_DEV void gemm_tile2(const OperandView<T>& A, const OperandView<T>& B, const T
 // Two GEMMs that share A, fused with the gated activation:
 //   P1 = A * op(B1),  P2 = A * op(B2)  (both stored, rounded to T),  ACT = act(gate) * value
 // with (gate, value) = (P1, P2) when gate_first, else (P2, P1), evaluated from the ROUNDED P1 / P2
-// exactly as a separate activation kernel reading them back would.  The workgroup's BN columns are
-// BN/2 columns of B1 followed by the same BN/2 columns of B2 (OperandView::half of `B`): waves
-// with wn < WAVES_N/2 accumulate P1, the others P2, and wave w pairs with wave w ^ (WAVES_N/2).
-// Per 32-row band every wave stages its fp32 results in LDS; after a barrier each wave of a pair
-// finishes 16 of the band's rows: reads both stagings, rounds, applies the activation and stores
-// the three outputs as 16-byte accesses.  Needs K % 64 == 0, Nh % 8 == 0, 16-byte aligned rows.
+// exactly as a separate activation kernel reading them back would.  The workgroup covers BN/2
+// columns of each product.  Needs K % 64 == 0, Nh % 8 == 0, 16-byte aligned rows.
 template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_MN, bool B_MN, bool B_DUAL = false>
 FX_DEV void gemm_mainloop32(const OperandView<T>& A, const OperandView<T>& B, int K, T* smem,
                             f32x16_t (&acc)[BM / WAVES_M / 32][BN / WAVES_N / 32]);
 
 // K32: the K loop with 32-wide steps over three stages (K % 32 == 0) instead of 64-wide over two.
+//
+// Each wave's B rows are WN/2 columns of B1 followed by the same WN/2 columns of B2
+// (OperandView::half = WN/2), so a wave holds both pre-activations of its rows x WN/2 columns and
+// needs nothing from any other wave.  Per 32-row band it stages the two blocks, rounded to T, in
+// its own LDS region and reads them back so that a lane holds 8 consecutive elements of one row of
+// each: the activation is computed from the rounded values (as the separate kernel would from
+// memory) and the three outputs leave as 16-byte stores, full 128-byte row segments.
+template <typename T, int NW, int WN>
+constexpr size_t glu_epilogue_lds_bytes() { return (size_t)NW * 2 * 32 * (WN / 2 + 8) * sizeof(T); }
+
 template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool B_MN, int ACT, bool K32 = false>
 FX_DEV void gemm_tile2_glu(const OperandView<T>& A, const OperandView<T>& B, T* P1, T* P2, int64_t ldp, T* ACTO,
                            int64_t ldact, int M, int Nh, int K, bool gate_first, T* smem) {
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     constexpr int TM = WM / 32, TN = WN / 32;
-    constexpr int HW = WAVES_N / 2;                 // waves per half along n
-    constexpr int PITCH = WN + 4, GROUPS = WN / 8;
-    constexpr int PER_LANE = 16 * GROUPS / 64;
-    static_assert(WAVES_N % 2 == 0 && (16 * GROUPS) % 64 == 0, "unsupported wave layout for the gated epilogue");
+    constexpr int HC = WN / 2;                       // columns of each output per wave
+    constexpr int PITCH = HC + 8;                    // staged row pitch in elements: rows stay 16-byte aligned
+    constexpr int GROUPS = HC / 8, PER_LANE = 32 * GROUPS / 64;
+    static_assert(TN % 2 == 0 && HC % 32 == 0 && (32 * GROUPS) % 64 == 0, "unsupported wave layout for the gated epilogue");
+    typedef typename VecOf<T>::type Pack;
+    typedef T t4_t __attribute__((ext_vector_type(4)));
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
     f32x16_t acc[TM][TN];
     if constexpr (K32) gemm_mainloop32<T, BM, BN, WAVES_M, WAVES_N, false, B_MN, true>(A, B, K, smem, acc);
     else gemm_mainloop2<T, BM, BN, WAVES_M, WAVES_N, false, B_MN, true>(A, B, K, smem, acc);
 
-    float* stage = reinterpret_cast<float*>(smem) + wave * 32 * PITCH;
-    const bool second = wn >= HW;
-    const float* s1 = reinterpret_cast<float*>(smem) + (second ? wave - HW : wave) * 32 * PITCH;
-    const float* s2 = s1 + HW * 32 * PITCH;
-    const int row_base = A.origin + wm * WM, col_base = B.origin + (wn % HW) * WN;
+    T* st1 = smem + wave * (2 * 32 * PITCH);
+    T* st2 = st1 + 32 * PITCH;
+    const int row_base = A.origin + wm * WM, col_base = B.origin + wn * HC;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
+        for (int j = 0; j < TN; ++j) {
+            T* dst = (j < TN / 2 ? st1 : st2) + (lane & 31) * PITCH + (j % (TN / 2)) * 32 + 4 * (lane >> 5);
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                const f32x4_t q = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
-                *reinterpret_cast<f32x4_t*>(stage + (lane & 31) * PITCH + j * 32 + 8 * g + 4 * (lane >> 5)) = q;
+                const t4_t q = {(T)acc[i][j][4 * g], (T)acc[i][j][4 * g + 1], (T)acc[i][j][4 * g + 2], (T)acc[i][j][4 * g + 3]};
+                *reinterpret_cast<t4_t*>(dst + 8 * g) = q;
             }
-        __syncthreads();
+        }
+        // a wave reads back only what it wrote itself; its LDS accesses complete in order
 #pragma unroll
         for (int t = 0; t < PER_LANE; ++t) {
             const int id = t * 64 + lane;
-            const int rr = (second ? 16 : 0) + id / GROUPS, cg = id % GROUPS;
+            const int rr = id / GROUPS, cg = id % GROUPS;
             const int row = row_base + i * 32 + rr, col = col_base + cg * 8;
             if (row < M && col < Nh) {
-                const f32x4_t a0 = *reinterpret_cast<const f32x4_t*>(s1 + rr * PITCH + cg * 8);
-                const f32x4_t a1 = *reinterpret_cast<const f32x4_t*>(s1 + rr * PITCH + cg * 8 + 4);
-                const f32x4_t b0 = *reinterpret_cast<const f32x4_t*>(s2 + rr * PITCH + cg * 8);
-                const f32x4_t b1 = *reinterpret_cast<const f32x4_t*>(s2 + rr * PITCH + cg * 8 + 4);
-                float v1[8], v2[8], y[8];
+                const Pack p1 = *reinterpret_cast<const Pack*>(st1 + rr * PITCH + cg * 8);
+                const Pack p2 = *reinterpret_cast<const Pack*>(st2 + rr * PITCH + cg * 8);
+                Pack y;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    v1[e] = round_to<T>(a0[e]); v1[4 + e] = round_to<T>(a1[e]);
-                    v2[e] = round_to<T>(b0[e]); v2[4 + e] = round_to<T>(b1[e]);
+                for (int e = 0; e < 8; ++e) {
+                    const float v1 = (float)p1[e], v2 = (float)p2[e];
+                    y[e] = (T)(gate_first ? glu_fwd_elem<T, ACT>(v1, v2) : glu_fwd_elem<T, ACT>(v2, v1));
                 }
-#pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    y[e] = gate_first ? glu_fwd_elem<T, ACT>(v1[e], v2[e]) : glu_fwd_elem<T, ACT>(v2[e], v1[e]);
-                store_f32<T, 8>(P1 + (int64_t)row * ldp + col, v1);
-                store_f32<T, 8>(P2 + (int64_t)row * ldp + col, v2);
-                store_f32<T, 8>(ACTO + (int64_t)row * ldact + col, y);
+                *reinterpret_cast<Pack*>(P1 + (int64_t)row * ldp + col) = p1;
+                *reinterpret_cast<Pack*>(P2 + (int64_t)row * ldp + col) = p2;
+                *reinterpret_cast<Pack*>(ACTO + (int64_t)row * ldact + col) = y;
             }
         }
-        __syncthreads();
     }
+}
+
+// LDS bytes of a workgroup of the gated tile: its K-loop stages or its epilogue staging.
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool K32>
+constexpr size_t gemm2_glu_lds_bytes() {
+    constexpr size_t tiles = (size_t)(K32 ? 3 * 32 : 2 * GEMM_BK) * (BM + BN) * sizeof(T);
+    constexpr size_t epi = glu_epilogue_lds_bytes<T, WAVES_M * WAVES_N, BN / WAVES_N>();
+    return tiles > epi ? tiles : epi;
 }
 
 // ---------------------------------------------------------------- 32-wide K-steps, three LDS stages
@@ -604,8 +614,8 @@ FX_DEV void tile32_load_direct(const OperandView<T>& op, int k0, T* lds, int wav
 #pragma unroll
     for (int j = 0; j < NI; ++j) {
         const int r = (j * NW + wave) * 16 + rr;
-        const bool second = DUAL && r >= op.half;
-        int g = op.origin + (second ? r - op.half : r);
+        const bool second = DUAL && op.dual_second(r);
+        int g = op.origin + (DUAL ? op.dual_index(r) : r);
         g = g < op.ext ? g : op.ext - 1;
         const int c = pos ^ swz_k<32>(r);
         load_to_lds16((second ? op.base2 : op.base) + (int64_t)g * op.ld + k0 + c * 8, lds + (j * NW + wave) * 16 * 32);
@@ -624,8 +634,8 @@ FX_DEV void tile32_load_direct_tr(const OperandView<T>& op, int k0, T* lds, int 
         const int q = j * NW + wave;
         const int k = q * KPI + kin;
         const int c = pos ^ (swz_tr(k) % CPR);
-        const bool second = DUAL && c * 8 >= op.half;
-        int g = op.origin + (second ? c * 8 - op.half : c * 8);
+        const bool second = DUAL && op.dual_second(c * 8);
+        int g = op.origin + (DUAL ? op.dual_index(c * 8) : c * 8);
         g = g + 8 <= op.ext ? g : op.ext - 8;
         load_to_lds16((second ? op.base2 : op.base) + (int64_t)(k0 + k) * op.ld + g, lds + q * 512);
     }

@@ -3,7 +3,8 @@
 // The reference runs two GEMMs (x1 = h W_1, x3 = h W_3, both saved for the backward pass) and
 // then a gated-activation kernel that reads them back (flextrain/nn/blocks/ffn_dense.py:130-146).
 // Here a workgroup accumulates the same 128 columns of both products from one pass over its rows
-// of h, stores x1 and x3 and, from their rounded values, act(x1) * x3: the activation costs no
+// of h (each wave the same 64 columns of both), stores x1 and x3 and, from their rounded values,
+// act(x1) * x3: the activation costs no
 // extra pass over HBM and h is read once.  Results are those of the three separate launches.
 #include "gemm_core2.h"
 #include "flexhip.h"
@@ -18,8 +19,8 @@ __global__ __launch_bounds__(512) void gemm_dual_glu_kernel(
     int tm, tn;
     tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
     OperandView<T> a{A, lda, M, tm * 256};
-    OperandView<T> b{B1, ldb, Nh, tn * 128, 128, B2};
-    gemm_tile2_glu<T, 256, 256, 2, 4, B_MN, ACT>(a, b, P1, P2, ldp, ACTO, ldact, M, Nh, K, gate_first != 0,
+    OperandView<T> b{B1, ldb, Nh, tn * 128, 64, B2};     // 4 x 2 waves of 64 x 128: 64 columns of each product per wave
+    gemm_tile2_glu<T, 256, 256, 4, 2, B_MN, ACT>(a, b, P1, P2, ldp, ACTO, ldact, M, Nh, K, gate_first != 0,
                                                  reinterpret_cast<T*>(smem_raw));
 }
 
@@ -27,7 +28,7 @@ template <typename T, bool B_MN, int ACT>
 static void launch_dual(const void* A, int64_t lda, const void* B1, const void* B2, int64_t ldb, void* P1, void* P2,
                         int64_t ldp, void* act, int64_t ldact, int M, int Nh, int K, int gate_first, hipStream_t s) {
     auto kern = gemm_dual_glu_kernel<T, B_MN, ACT>;
-    constexpr size_t lds = gemm2_lds_bytes<T, 256, 256, 2, 4>();
+    constexpr size_t lds = gemm2_glu_lds_bytes<T, 256, 256, 4, 2, false>();
     FX_ENSURE_DYNAMIC_LDS(kern, lds);
     const int tiles_m = (M + 255) / 256, tiles_n = (Nh + 127) / 128;
     kern<<<dim3((unsigned)(tiles_m * tiles_n)), 512, lds, s>>>(

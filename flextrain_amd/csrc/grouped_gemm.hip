@@ -147,7 +147,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64, K32 ? 2 : 1) void grouped_r
     const int rows = OFFSETS[e + 1] - OFFSETS[e];
     OperandView<T> a{A + row0 * lda, lda, rows, m0};
     const T* b1 = B + (int64_t)e * b_expert_stride;
-    OperandView<T> b{b1, ldb, Nh, tn * (BN / 2), BN / 2, b1 + b2_delta};
+    OperandView<T> b{b1, ldb, Nh, tn * (BN / 2), BN / WAVES_N / 2, b1 + b2_delta};
     gemm_tile2_glu<T, BM, BN, WAVES_M, WAVES_N, B_MN, ACT_SILU, K32>(a, b, P1 + row0 * ldp, P2 + row0 * ldp, ldp,
                                                                      ACTO + row0 * ldact, ldact, rows, Nh, K,
                                                                      gate_first != 0, smem);
@@ -268,8 +268,7 @@ extern "C" int fx_grouped_gemm_rows_glu(const void* A, int64_t lda, const void* 
 #define FX_GLU(TT, BM_, BN_, WM_, WN_, BMN, K32_)                                                         \
     {                                                                                                     \
         auto kern = grouped_rows_glu_kernel<TT, BM_, BN_, WM_, WN_, BMN, K32_>;                           \
-        constexpr size_t lds = K32_ ? gemm32_lds_bytes<TT, BM_, BN_, WM_, WN_>()                          \
-                                    : gemm2_lds_bytes<TT, BM_, BN_, WM_, WN_>();                          \
+        constexpr size_t lds = gemm2_glu_lds_bytes<TT, BM_, BN_, WM_, WN_, K32_>();                       \
         FX_ENSURE_DYNAMIC_LDS(kern, lds);                                                                 \
         const int tiles_n = cdiv_i(Nh, BN_ / 2);                                                          \
         kern<<<dim3(max_tiles * (unsigned)tiles_n), WM_ * WN_ * 64, lds, stream>>>(                       \
@@ -279,7 +278,7 @@ extern "C" int fx_grouped_gemm_rows_glu(const void* A, int64_t lda, const void* 
     }
     // 128-row tiles: 128 x 256 (128 columns of each half) with 32-wide K-steps, two workgroups per CU
 #define FX_GLU_T(TT)                                                                                      \
-    if (BM == 256) { if (trans_b) FX_GLU(TT, 256, 256, 2, 4, false, false) else FX_GLU(TT, 256, 256, 2, 4, true, false) } \
+    if (BM == 256) { if (trans_b) FX_GLU(TT, 256, 256, 4, 2, false, false) else FX_GLU(TT, 256, 256, 4, 2, true, false) } \
     else { if (trans_b) FX_GLU(TT, 128, 256, 2, 2, false, true) else FX_GLU(TT, 128, 256, 2, 2, true, true) }
     if (dt == DT_BF16) { FX_GLU_T(bf16) } else { FX_GLU_T(f16) }
 #undef FX_GLU_T
