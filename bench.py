@@ -153,6 +153,20 @@ def run_rmsnorm(torch, ops, dev, stream, rn):
     rows.append(_op_entry("c1.rmsnorm_bwd(dX+=,dW+=,y)", 5 * T * D * 2 + D * 2 + T * 4 + 2 * D * 4, "GB/s", ms))
     del sets, fwd, bwd, bwd_e
     torch.cuda.empty_cache()
+    # ---- the same kernels at the token count of the headline workload's layer input x 4 (32768 rows, 268 MB per
+    # tensor): configs[0] is 16 MB per tensor and therefore bound by launch and latency, not by HBM
+    T2 = 32768
+    big = [dict(x=rn(T2, D).to(dev), dy=rn(T2, D).to(dev), y=torch.empty(T2, D, dtype=torch.bfloat16, device=dev),
+                dx=torch.zeros(T2, D, dtype=torch.bfloat16, device=dev), rstd=torch.empty(T2, 1, dtype=torch.float32, device=dev))
+           for _ in range(3)]
+    fwd = [lambda s=s: ops.flextrain_rmsnorm_fwd(s["x"], w, output=s["y"], rstd=s["rstd"]) for s in big]
+    ms = _time_launches(torch, stream, fwd, warmup=3, reps=12)
+    rows.append(_op_entry("c1x16.rmsnorm_fwd at 32768 tokens", 2 * T2 * D * 2 + D * 2 + T2 * 4, "GB/s", ms))
+    bwd = [lambda s=s: ops.flextrain_rmsnorm_bwd(s["dy"], s["x"], w, s["rstd"], dX=s["dx"], dW=dw) for s in big]
+    ms = _time_launches(torch, stream, bwd, warmup=3, reps=12)
+    rows.append(_op_entry("c1x16.rmsnorm_bwd(dX+=,dW+=) at 32768 tokens", 4 * T2 * D * 2 + D * 2 + T2 * 4 + 2 * D * 4, "GB/s", ms))
+    del big, fwd, bwd
+    torch.cuda.empty_cache()
     return rows
 
 
