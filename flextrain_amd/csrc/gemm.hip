@@ -158,6 +158,7 @@ static bool mfma_ok(const void* A, const void* B, int M, int N, int K, int64_t l
     if (d_dt != a_dt && !(a_dt == DT_BF16 && d_dt == DT_F32)) return false;
     if (has_c && c_dt != d_dt) return false;
     if (!aligned16(A) || !aligned16(B) || (lda & 7) || (ldb & 7)) return false;
+    if (lda >= (1 << 23) || ldb >= (1 << 23)) return false;   // 32-bit per-lane byte offsets inside a tile
     if (ta ? (M & 7) : (K & 7)) return false;
     if (tb ? (K & 7) : (N & 7)) return false;
     return true;

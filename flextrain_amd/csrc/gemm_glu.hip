@@ -47,6 +47,7 @@ extern "C" int fx_gemm_dual_glu(const void* A, int64_t lda, const void* B1, cons
     if (M == 0) return 0;
     if (!A || !B1 || !B2 || !P1 || !P2 || !act) FX_FAIL("fx_gemm_dual_glu: null pointer");
     if (dt != DT_BF16 && dt != DT_F16) FX_FAIL("fx_gemm_dual_glu: bf16 or fp16 only");
+    if (lda >= (1 << 23) || ldb >= (1 << 23)) FX_FAIL("fx_gemm_dual_glu: leading dimensions must be below 2^23 elements");
     if (activation != ACT_SILU && activation != ACT_GELU_TANH) FX_FAIL("fx_gemm_dual_glu: unknown activation %d", activation);
     if ((K & 63) || (Nh & 7) || (lda & 7) || (ldb & 7) || (ldp & 7) || (ldact & 7) || !aligned16(A) || !aligned16(B1) ||
         !aligned16(B2) || !aligned16(P1) || !aligned16(P2) || !aligned16(act))

@@ -201,6 +201,7 @@ extern "C" int fx_grouped_gemm_rows(const void* A, int64_t lda, const void* B, i
     if (!A || !B || !D || !counts) FX_FAIL("fx_grouped_gemm_rows: null pointer");
     if (!ws || ws_bytes < fx_grouped_ws_bytes(E, total_rows)) FX_FAIL("fx_grouped_gemm_rows: workspace too small");
     if (dt != DT_BF16 && dt != DT_F16) FX_FAIL("fx_grouped_gemm_rows: bf16 or fp16 only");
+    if (lda >= (1 << 23) || ldb >= (1 << 23)) FX_FAIL("fx_grouped_gemm_rows: leading dimensions must be below 2^23 elements");
     if (!aligned16(A) || !aligned16(B) || !aligned16(D) || (lda & 7) || (ldb & 7) || (K & 7) || (b_expert_stride & 7) ||
         (!trans_b && (N & 7)))
         FX_FAIL("fx_grouped_gemm_rows: operands must be 16-byte aligned with K (and N when B is (K,N)) a multiple of 8");
@@ -257,6 +258,7 @@ extern "C" int fx_grouped_gemm_rows_glu(const void* A, int64_t lda, const void* 
     if (!A || !B || !P1 || !P2 || !act || !counts) FX_FAIL("fx_grouped_gemm_rows_glu: null pointer");
     if (!ws || ws_bytes < fx_grouped_ws_bytes(E, total_rows)) FX_FAIL("fx_grouped_gemm_rows_glu: workspace too small");
     if (dt != DT_BF16 && dt != DT_F16) FX_FAIL("fx_grouped_gemm_rows_glu: bf16 or fp16 only");
+    if (lda >= (1 << 23) || ldb >= (1 << 23)) FX_FAIL("fx_grouped_gemm_rows_glu: leading dimensions must be below 2^23 elements");
     if (!aligned16(A) || !aligned16(B) || !aligned16(P1) || !aligned16(P2) || !aligned16(act) || (lda & 7) || (ldb & 7) ||
         (ldp & 7) || (ldact & 7) || (K & 63) || (Nh & 7) || (b_expert_stride & 7) || (b2_delta & 7))
         FX_FAIL("fx_grouped_gemm_rows_glu: needs K %% 64 == 0, N %% 8 == 0, strides %% 8 == 0 and 16-byte aligned operands");
@@ -295,6 +297,7 @@ extern "C" int fx_grouped_gemm_wgrad(const void* A, int64_t lda, const void* B, 
     if (!A || !B || !G || !counts) FX_FAIL("fx_grouped_gemm_wgrad: null pointer");
     if (!ws || ws_bytes < fx_grouped_ws_bytes(E, total_rows)) FX_FAIL("fx_grouped_gemm_wgrad: workspace too small");
     if (dt != DT_BF16 && dt != DT_F16) FX_FAIL("fx_grouped_gemm_wgrad: bf16 or fp16 only");
+    if (lda >= (1 << 23) || ldb >= (1 << 23)) FX_FAIL("fx_grouped_gemm_wgrad: leading dimensions must be below 2^23 elements");
     if (g_dt != dt && !(dt == DT_BF16 && g_dt == DT_F32)) FX_FAIL("fx_grouped_gemm_wgrad: G must match the inputs or be fp32 (bf16 inputs)");
     if (!aligned16(A) || !aligned16(B) || (lda & 7) || (ldb & 7) || (M & 7) || (N & 7))
         FX_FAIL("fx_grouped_gemm_wgrad: operands must be 16-byte aligned with M and N multiples of 8");
