@@ -696,6 +696,62 @@ FX_DEV void tile32_load_direct_tr(const OperandView<T>& op, int k0, T* lds, int 
     }
 }
 
+// The 32-wide tiles with a wave-uniform base and 32-bit lane offsets (see TileLoader); the
+// M/N-contiguous two-matrix tile keeps the function form above.
+template <typename T, int ROWS, int NW, bool MN, bool DUAL>
+struct Tile32Loader {
+    static constexpr int CPR = ROWS / 8;                      // M/N-contiguous: 16-byte chunks per LDS row
+    static constexpr int KPI = 64 / (CPR > 64 ? 64 : CPR);    //                 k-rows per instruction
+    static constexpr int NI = MN ? 32 / KPI / NW : ROWS / 16 / NW;
+    static_assert(!(MN && DUAL), "a two-matrix M/N-contiguous tile mixes both matrices inside one instruction");
+    static_assert(MN ? ((ROWS == 128 || ROWS == 256) && (32 / KPI) % NW == 0) : ROWS % (16 * NW) == 0, "unsupported tile rows");
+    unsigned off[NI];
+    const T* base;
+    const T* base2;
+    int64_t step;
+    int half;
+
+    FX_DEV void init(const OperandView<T>& op, int wave, int lane) {
+        half = op.half;
+        if (!MN) {
+            const int rr = lane >> 2, pos = lane & 3;
+#pragma unroll
+            for (int j = 0; j < NI; ++j) {
+                const int r = (j * NW + wave) * 16 + rr;
+                int g = op.origin + (DUAL ? op.dual_index(r) : r);
+                g = g < op.ext ? g : op.ext - 1;
+                off[j] = (unsigned)(((int64_t)(g - op.origin) * op.ld + (pos ^ swz_k<32>(r)) * 8) * (int64_t)sizeof(T));
+            }
+            base = op.base + (int64_t)op.origin * op.ld;
+            base2 = DUAL ? op.base2 + (int64_t)op.origin * op.ld : nullptr;
+            step = 32;
+        } else {
+            const int kin = lane / CPR, pos = lane % CPR;
+#pragma unroll
+            for (int j = 0; j < NI; ++j) {
+                const int k = (j * NW + wave) * KPI + kin;
+                const int c = pos ^ (swz_tr(k) % CPR);
+                int g = op.origin + c * 8;
+                g = g + 8 <= op.ext ? g : op.ext - 8;
+                off[j] = (unsigned)(((int64_t)k * op.ld + (g - op.origin)) * (int64_t)sizeof(T));
+            }
+            base = op.base + op.origin;
+            base2 = nullptr;
+            step = (int64_t)32 * op.ld;
+        }
+    }
+    template <int J>
+    FX_DEV void issue(T* lds, int wave) {
+        const unsigned lds_addr = (unsigned)(uintptr_t)(lds + (J * NW + wave) * 512);
+        const T* b = (DUAL && ((((J * NW + wave) * 16) & half) != 0)) ? base2 : base;
+        load_to_lds16_s(off[J], b, lds_addr);
+        if (J == NI - 1) {
+            base += step;
+            if (DUAL) base2 += step;
+        }
+    }
+};
+
 template <typename T, int BM, int BN, int WAVES_M, int WAVES_N>
 constexpr size_t gemm32_lds_bytes() {
     constexpr size_t tiles = (size_t)3 * (BM + BN) * 32 * sizeof(T);
@@ -714,7 +770,7 @@ FX_DEV void gemm_mainloop32(const OperandView<T>& A, const OperandView<T>& B, in
     constexpr int STAGE = (BM + BN) * 32;
     constexpr int LD = (BM + BN) * 64 / 1024 / NW;      // load instructions per wave per K-step
     static_assert((BM + BN) * 64 % (1024 * NW) == 0, "loads must split evenly over the waves");
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -723,11 +779,20 @@ FX_DEV void gemm_mainloop32(const OperandView<T>& A, const OperandView<T>& B, in
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
     const int n = K / 32;
-    auto issue = [&](int kt, T* buf) {
-        if (!A_MN) tile32_load_direct<T, BM, NW>(A, kt * 32, buf, wave, lane);
-        else tile32_load_direct_tr<T, BM, NW>(A, kt * 32, buf, wave, lane);
-        if (!B_MN) tile32_load_direct<T, BN, NW, B_DUAL>(B, kt * 32, buf + BM * 32, wave, lane);
-        else tile32_load_direct_tr<T, BN, NW, B_DUAL>(B, kt * 32, buf + BM * 32, wave, lane);
+    constexpr bool B_FN = B_MN && B_DUAL;                 // the one tile form without a scalar-base loader
+    typedef Tile32Loader<T, BM, NW, A_MN, false> LoadA;
+    typedef Tile32Loader<T, BN, NW, B_MN, B_DUAL && !B_FN> LoadB;
+    static_assert(LoadA::NI + LoadB::NI == LD, "load instruction count");
+    LoadA la;
+    LoadB lb;
+    la.init(A, wave, lane);
+    if constexpr (!B_FN) lb.init(B, wave, lane);
+    int kb = 0;                                           // next K-step of the function-form B loader
+    // K-steps are issued in order, each exactly once
+    auto issue = [&](T* buf) {
+        static_for<0, LoadA::NI>([&](auto j) { la.template issue<decltype(j)::value>(buf, wave); });
+        if constexpr (B_FN) tile32_load_direct_tr<T, BN, NW, true>(B, (kb++) * 32, buf + BM * 32, wave, lane);
+        else static_for<0, LoadB::NI>([&](auto j) { lb.template issue<decltype(j)::value>(buf + BM * 32, wave); });
     };
     if (n > 0) {
         typedef MmaPipe<T, BM, BN, WM, WN, A_MN, B_MN, 32> Pipe;
@@ -736,15 +801,15 @@ FX_DEV void gemm_mainloop32(const OperandView<T>& A, const OperandView<T>& B, in
         T* cur = smem;
         T* nxt = smem + STAGE;
         T* aft = smem + 2 * STAGE;
-        issue(0, cur);
+        issue(cur);
         if (n > 1) {
-            issue(1, nxt);
+            issue(nxt);
             asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LD) : "memory");   // step 0 landed, step 1 may be in flight
         } else {
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         }
         __syncthreads();
-        if (n > 2) issue(2, aft);
+        if (n > 2) issue(aft);
         Pipe::fetch_all(f0, cur, cur + BM * 32, 0, ra, rb, lane);
         for (int kt = 0; kt + 1 < n; ++kt) {
             Pipe::template sub<true>(acc, f0, f1, cur, cur + BM * 32, 1, ra, rb, lane);
@@ -752,7 +817,7 @@ FX_DEV void gemm_mainloop32(const OperandView<T>& A, const OperandView<T>& B, in
             if (kt + 2 < n) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(LD) : "memory");
             else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
             __syncthreads();
-            if (kt + 3 < n) issue(kt + 3, cur);          // `cur` is free for everyone now
+            if (kt + 3 < n) issue(cur);                  // `cur` is free for everyone now
             Pipe::template sub<true>(acc, f1, f0, nxt, nxt + BM * 32, 0, ra, rb, lane);
             T* t = cur; cur = nxt; nxt = aft; aft = t;
         }
