@@ -509,10 +509,16 @@ FX_DEV void gemm_mainloop2(const OperandView<T>& A, const OperandView<T>& B, int
         auto issue = [&](T* buf) { static_for<0, LD>([&](auto idx) { issue_one(idx, buf); }); };
         typename Pipe::Slot f0, f1;
         const int ra = wm * WM, rb = wn * WN;
+        // both buffers are free at the start of a tile: the first two K-steps go out together and
+        // only the first is waited for (short-K tiles spend a visible share of their time here)
         issue(smem);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (nfull > 1) {
+            issue(smem + BUF);
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LD) : "memory");
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
         __syncthreads();
-        if (nfull > 1) issue(smem + BUF);
         Pipe::fetch_all(f0, smem, smem + BM * GEMM_BK, 0, ra, rb, lane);
         for (int kt = 0; kt + 1 < nfull; ++kt) {
             T* cur = smem + (kt & 1) * BUF;
