@@ -394,6 +394,64 @@ FX_DEV void epilogue_tile(f32x16_t (&acc)[WM / 32][WN / 32], const TD* C, TD* D,
     // staged: one exposed memory round trip per group instead of one per band and lane slot (a
     // short-K tile spends as long in its epilogue as in its K loop otherwise).  A group is as many
     // bands as fit 64 registers per lane.
+#ifndef FX_EPI_MODE
+#define FX_EPI_MODE 0
+#endif
+    if constexpr (sizeof(TD) == 2 && FX_EPI_MODE == 2) {
+        if (beta == 0.f && (ldd & 3) == 0 && (reinterpret_cast<uintptr_t>(D) & 7u) == 0) {
+            typedef TD TD4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const int row = row_base + i * 32 + (lane & 31), col = col_base + j * 32 + 8 * g + 4 * (lane >> 5);
+                        if (row >= M) continue;
+                        TD4 v;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] = (TD)(alpha * acc[i][j][4 * g + e]);
+                        TD* dst = D + (int64_t)row * ldd + col;
+                        if (col + 4 <= N) *reinterpret_cast<TD4*>(dst) = v;
+                        else
+                            for (int e = 0; e < 4 && col + e < N; ++e) dst[e] = v[e];
+                    }
+            return;
+        }
+    }
+    if constexpr (sizeof(TD) == 2 && FX_EPI_MODE == 1) {
+        if (beta == 0.f && vec_ok) {
+            typedef TD TD4 __attribute__((ext_vector_type(4)));
+            typedef typename VecOf<TD>::type TD8;
+            constexpr int PT = WN + 8;
+            TD* st = reinterpret_cast<TD*>(smem) + wave * 32 * PT;
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        TD4 v;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] = (TD)(alpha * acc[i][j][4 * g + e]);
+                        *reinterpret_cast<TD4*>(st + (lane & 31) * PT + j * 32 + 8 * g + 4 * (lane >> 5)) = v;
+                    }
+#pragma unroll
+                for (int t = 0; t < PER_LANE; ++t) {
+                    const int id = t * 64 + lane;
+                    const int rr = id / GROUPS, cg = id % GROUPS;
+                    const int row = row_base + i * 32 + rr, col = col_base + cg * 8;
+                    if (row >= M || col >= N) continue;
+                    const TD8 v = *reinterpret_cast<const TD8*>(st + rr * PT + cg * 8);
+                    TD* dst = D + (int64_t)row * ldd + col;
+                    if (col + 8 <= N) *reinterpret_cast<TD8*>(dst) = v;
+                    else
+                        for (int e = 0; e < 8 && col + e < N; ++e) dst[e] = v[e];
+                }
+            }
+            return;
+        }
+    }
     typedef typename VecOf<TD>::type CV;
     constexpr int CVN = 8 / VecOf<TD>::N;                                   // 16-byte vectors per 8 elements
     constexpr int CB = (CVN == 1 || TM == 1) ? TM : TM / 2;                 // bands per prefetch group
@@ -489,6 +547,9 @@ FX_DEV void gemm_mainloop2(const OperandView<T>& A, const OperandView<T>& B, int
 
     const int nfull = K / GEMM_BK;  // K-steps that need no zero fill
     static_assert(GEMM_BK == 64, "the pipeline below is written out for four sub-steps per K-step");
+    // wave-uniform: does any element of this wave's sub-tile lie inside the matrices?
+    const bool live = __builtin_amdgcn_readfirstlane(
+        (A.origin + wm * WM < A.ext) && (B_DUAL || B.origin + wn * WN < B.ext));
     if (nfull > 0) {
         typedef MmaPipe<T, BM, BN, WM, WN, A_MN, B_MN> Pipe;
         typedef TileLoader<T, BM, NW, A_MN, false> LoadA;
@@ -519,6 +580,16 @@ FX_DEV void gemm_mainloop2(const OperandView<T>& A, const OperandView<T>& B, int
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         }
         __syncthreads();
+        if (!live) {
+            // no row (or column) of this wave's sub-tile exists: it keeps loading its share of the
+            // stages and meets every barrier of the loop below, and leaves the matrix cores of its
+            // SIMD to the wave it shares them with (the last row tile of an expert is mostly this)
+            for (int kt = 0; kt + 1 < nfull; ++kt) {
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();
+                if (kt + 2 < nfull) issue(smem + (kt & 1) * BUF);
+            }
+        } else {
         Pipe::fetch_all(f0, smem, smem + BM * GEMM_BK, 0, ra, rb, lane);
         for (int kt = 0; kt + 1 < nfull; ++kt) {
             T* cur = smem + (kt & 1) * BUF;
@@ -548,6 +619,7 @@ FX_DEV void gemm_mainloop2(const OperandView<T>& A, const OperandView<T>& B, int
             Pipe::template sub<true>(acc, f0, f1, cur, curb, 3, ra, rb, lane);
             Pipe::template sub<false>(acc, f1, f0, cur, curb, 0, ra, rb, lane);
         }
+        }
     }
     if (!B_DUAL && nfull * GEMM_BK < K) {  // K tail: through registers into the K-contiguous layout, zero-filled past K
         Staged2<BM, NT> sa;
@@ -558,7 +630,7 @@ FX_DEV void gemm_mainloop2(const OperandView<T>& A, const OperandView<T>& B, int
         stage2_store<T, BM, NT, A_MN>(sa, buf, tid);     // `buf` was last read two steps ago
         stage2_store<T, BN, NT, B_MN>(sb, buf + BM * GEMM_BK, tid);
         __syncthreads();
-        mma_step<T, BM, BN, WM, WN, false, false>(buf, buf + BM * GEMM_BK, wm * WM, wn * WN, lane, acc);
+        if (live) mma_step<T, BM, BN, WM, WN, false, false>(buf, buf + BM * GEMM_BK, wm * WM, wn * WN, lane, acc);
     }
     __syncthreads();  // every wave is past its last LDS read: the buffers become epilogue staging
     static_assert(gemm2_lds_bytes<T, BM, BN, WAVES_M, WAVES_N>() <= 160 * 1024, "tile configuration exceeds the 160 KB of LDS");
