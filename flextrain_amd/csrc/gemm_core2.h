@@ -394,64 +394,6 @@ FX_DEV void epilogue_tile(f32x16_t (&acc)[WM / 32][WN / 32], const TD* C, TD* D,
     // staged: one exposed memory round trip per group instead of one per band and lane slot (a
     // short-K tile spends as long in its epilogue as in its K loop otherwise).  A group is as many
     // bands as fit 64 registers per lane.
-#ifndef FX_EPI_MODE
-#define FX_EPI_MODE 0
-#endif
-    if constexpr (sizeof(TD) == 2 && FX_EPI_MODE == 2) {
-        if (beta == 0.f && (ldd & 3) == 0 && (reinterpret_cast<uintptr_t>(D) & 7u) == 0) {
-            typedef TD TD4 __attribute__((ext_vector_type(4)));
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-#pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        const int row = row_base + i * 32 + (lane & 31), col = col_base + j * 32 + 8 * g + 4 * (lane >> 5);
-                        if (row >= M) continue;
-                        TD4 v;
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) v[e] = (TD)(alpha * acc[i][j][4 * g + e]);
-                        TD* dst = D + (int64_t)row * ldd + col;
-                        if (col + 4 <= N) *reinterpret_cast<TD4*>(dst) = v;
-                        else
-                            for (int e = 0; e < 4 && col + e < N; ++e) dst[e] = v[e];
-                    }
-            return;
-        }
-    }
-    if constexpr (sizeof(TD) == 2 && FX_EPI_MODE == 1) {
-        if (beta == 0.f && vec_ok) {
-            typedef TD TD4 __attribute__((ext_vector_type(4)));
-            typedef typename VecOf<TD>::type TD8;
-            constexpr int PT = WN + 8;
-            TD* st = reinterpret_cast<TD*>(smem) + wave * 32 * PT;
-#pragma unroll
-            for (int i = 0; i < TM; ++i) {
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-#pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        TD4 v;
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) v[e] = (TD)(alpha * acc[i][j][4 * g + e]);
-                        *reinterpret_cast<TD4*>(st + (lane & 31) * PT + j * 32 + 8 * g + 4 * (lane >> 5)) = v;
-                    }
-#pragma unroll
-                for (int t = 0; t < PER_LANE; ++t) {
-                    const int id = t * 64 + lane;
-                    const int rr = id / GROUPS, cg = id % GROUPS;
-                    const int row = row_base + i * 32 + rr, col = col_base + cg * 8;
-                    if (row >= M || col >= N) continue;
-                    const TD8 v = *reinterpret_cast<const TD8*>(st + rr * PT + cg * 8);
-                    TD* dst = D + (int64_t)row * ldd + col;
-                    if (col + 8 <= N) *reinterpret_cast<TD8*>(dst) = v;
-                    else
-                        for (int e = 0; e < 8 && col + e < N; ++e) dst[e] = v[e];
-                }
-            }
-            return;
-        }
-    }
     typedef typename VecOf<TD>::type CV;
     constexpr int CVN = 8 / VecOf<TD>::N;                                   // 16-byte vectors per 8 elements
     constexpr int CB = (CVN == 1 || TM == 1) ? TM : TM / 2;                 // bands per prefetch group
