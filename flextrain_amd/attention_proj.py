@@ -70,6 +70,16 @@ class GQAAttentionProjections:
     def _mm(self, A, B, D, C=None, beta=0.0):
         return self.dispatcher.matmul(_stream_ptr(A), A=A, B=B, C=C, D=D, alpha=1.0, beta=beta)
 
+    def _mm_shared(self, A, Bs, Ds, Cs=None, beta=0.0):
+        """Products that share ``A`` (key / value projections, their weight gradients): one launch
+        where the dispatcher offers it, since each alone is too small to fill the GPU."""
+        shared = getattr(self.dispatcher, "matmul_shared_a", None)
+        if shared is not None:
+            return shared(_stream_ptr(A), A, Bs, Ds, Cs=Cs, alpha=1.0, beta=beta)
+        for i, B in enumerate(Bs):
+            self._mm(A, B, Ds[i], C=None if Cs is None else Cs[i], beta=beta)
+        return Ds
+
     def _rope_freqs(self, device) -> torch.Tensor:
         """inv_freq of the configured RoPE, built once (attention.py:373-390)."""
         if self._inv_freq is None or self._inv_freq.device != device:
@@ -83,8 +93,7 @@ class GQAAttentionProjections:
         cfg = self.cfg
         xq2d, xk2d, xv2d = slot.xq.view(-1, cfg.attn_dim), slot.xk.view(-1, cfg.kv_dim), slot.xv.view(-1, cfg.kv_dim)
         self._mm(attn_norm_output, weights["w_q"], xq2d)
-        self._mm(attn_norm_output, weights["w_k"], xk2d)
-        self._mm(attn_norm_output, weights["w_v"], xv2d)
+        self._mm_shared(attn_norm_output, [weights["w_k"], weights["w_v"]], [xk2d, xv2d])
         if cfg.qkv_bias:
             xq2d.add_(weights["b_q"])
             xk2d.add_(weights["b_k"])
@@ -179,13 +188,21 @@ class GQAAttentionProjections:
     def bwd_accumulate_qkv_grads(self, attn_norm_output, grads, slot, *, skip_grads: frozenset = frozenset(),
                                  capture_xy: dict | None = None) -> None:
         """``g_v, g_k, g_q += attn_norm_output^T d{v,k,q}`` (attention.py:777-823)."""
+        todo = []
         for name, dy_key in (("g_v", "bwd_local_dv"), ("g_k", "bwd_local_dk"), ("g_q", "bwd_dq")):
             dy = slot.aux[dy_key]
             if name in skip_grads:
                 if capture_xy is not None:
                     capture_xy[name] = (attn_norm_output, dy)
             else:
-                self._mm(attn_norm_output.T, dy, grads[name], C=grads[name], beta=1.0)
+                todo.append((name, dy))
+        kv = [(n, dy) for n, dy in todo if n in ("g_v", "g_k")]
+        if len(kv) == 2:     # the two small products as one launch
+            g = [grads[n] for n, _ in kv]
+            self._mm_shared(attn_norm_output.T, [dy for _, dy in kv], g, Cs=g, beta=1.0)
+            todo = [t for t in todo if t[0] == "g_q"]
+        for name, dy in todo:
+            self._mm(attn_norm_output.T, dy, grads[name], C=grads[name], beta=1.0)
         del slot.aux["bwd_dq"]
         del slot.aux["bwd_local_dk"]
         del slot.aux["bwd_local_dv"]

@@ -95,6 +95,16 @@ static TileCfg choose_tile(int M, int N) {
 static int choose_splits(int M, int N, int K, size_t workspace_bytes) {
     const long tiles = (long)cdiv(M, 256) * cdiv(N, 256);
     if (tiles >= 128 || K < 1024) return 1;
+    // 128 x 128 tiles fill the GPU without a reduction pass over fp32 partial products, at about
+    // 1.05 instead of 1.25 PFLOP/s: the better choice unless K is long (key / value weight
+    // gradients, 4096 x 1024 with K = 8192: 87 against 104 us; LM-head dX with K = 128256: 1030
+    // against 890 us).  Times in microseconds.
+    if ((long)cdiv(M, 128) * cdiv(N, 128) >= 192) {
+        const double flops = 2.0 * M * N * (double)K;
+        const double slower_tiles_us = flops * (1.0 / 1.05e9 - 1.0 / 1.25e9);
+        const double reduce_us = 8.0 + (double)M * N * 4.0 * (256.0 / tiles + 1.0) / 4.0e6;
+        if (slower_tiles_us < reduce_us) return 1;
+    }
     long s = 256 / tiles;
     if (s > K / 512) s = K / 512;       // at least 8 K-steps per split
     const size_t per = (size_t)M * N * sizeof(float);

@@ -140,6 +140,75 @@ class CublasLtDispatcher:
         self.total_python_ns += time.perf_counter_ns() - t0
         return D
 
+    def matmul_shared_a(self, stream_ptr, A, Bs, Ds, Cs=None, alpha=1.0, beta=0.0):
+        """``Ds[i] = alpha * A @ Bs[i] + beta * Cs[i]`` for up to four ``Bs`` in ONE launch when the
+        operands allow it (bf16 / fp16, outputs of the input type, every ``B`` in the same
+        row- or column-major form, 16-byte aligned with multiples of 8 on the contiguous axes);
+        otherwise one :meth:`matmul` per product.  Same results either way.  No counterpart in
+        the reference, which calls ``matmul`` once per projection (attention.py:424-463): products
+        like the key / value projections are each too small to fill the GPU alone."""
+        n = len(Bs)
+        if len(Ds) != n or (Cs is not None and len(Cs) != n):
+            raise ValueError("matmul_shared_a: Bs, Ds and Cs must have the same length")
+        if self._segments_ok(A, Bs, Ds, Cs):
+            ptr_A, ld_A, trans_a = _get_layout(A)
+            lays = [_get_layout(b) for b in Bs]
+            M, K = A.shape
+            vp, i64 = ctypes.c_void_p * n, ctypes.c_int64 * n
+            b_ptrs, b_ld = vp(*[l[0] for l in lays]), i64(*[l[1] for l in lays])
+            d_ptrs, d_ld = vp(*[d.data_ptr() for d in Ds]), i64(*[d.stride(0) for d in Ds])
+            if Cs is not None and beta != 0.0:
+                c_ptrs, c_ld = vp(*[c.data_ptr() for c in Cs]), i64(*[c.stride(0) for c in Cs])
+            else:
+                c_ptrs, c_ld = None, None
+            ns = (ctypes.c_int * n)(*[b.shape[1] for b in Bs])
+            rc = self._lib.fx_gemm_segments(ptr_A, ld_A, trans_a, n, b_ptrs, b_ld, lays[0][2], c_ptrs, c_ld, d_ptrs,
+                                            d_ld, M, ns, K, alpha, beta, _dtype_to_enum[A.dtype], stream_ptr)
+            if rc != 0:
+                raise RuntimeError("fx_gemm_segments failed")
+            return Ds
+        for i in range(n):
+            self.matmul(stream_ptr, A, Bs[i], C=None if Cs is None else Cs[i], D=Ds[i], alpha=alpha, beta=beta)
+        return Ds
+
+    @staticmethod
+    def _segments_ok(A, Bs, Ds, Cs):
+        if not 2 <= len(Bs) <= 4 or A.dim() != 2 or A.dtype not in (torch.bfloat16, torch.float16):
+            return False
+        M, K = A.shape
+        if M == 0 or K == 0:
+            return False
+
+        def operand_ok(t, rows, cols):
+            if t.dim() != 2 or t.shape[0] != rows or t.dtype != A.dtype or t.data_ptr() % 16:
+                return False
+            sr, sc = t.stride()
+            if sc == 1:      # row-major: the columns are contiguous
+                return sr % 8 == 0 and sr < (1 << 23) and (cols is None or cols % 8 == 0) and t.shape[1] % 8 == 0
+            if sr == 1:      # column-major: the rows are contiguous
+                return sc % 8 == 0 and sc < (1 << 23) and rows % 8 == 0
+            return False
+
+        if not operand_ok(A, M, None):
+            return False
+        form = None
+        for i, b in enumerate(Bs):
+            if not operand_ok(b, K, None) or b.shape[1] <= 0:
+                return False
+            f = b.stride(1) == 1
+            if form is None:
+                form = f
+            if f != form:
+                return False
+            d = Ds[i]
+            if d.dim() != 2 or d.shape != (M, b.shape[1]) or d.dtype != A.dtype or d.stride(1) != 1:
+                return False
+            if Cs is not None:
+                c = Cs[i]
+                if c.dim() != 2 or c.shape != d.shape or c.dtype != A.dtype or c.stride(1) != 1:
+                    return False
+        return True
+
     def matmul_fast(self, stream_ptr, A, B, C=None, D=None, alpha=1.0, beta=0.0):
         """Hot-path variant: no validation, no allocation (``D`` required), no
         wrapper timing.  Bit-identical results to :meth:`matmul`."""

@@ -271,6 +271,21 @@ int fx_gemm_dual_glu(const void* A, int64_t lda, const void* B1, const void* B2,
                      void* P1, void* P2, int64_t ldp, void* act, int64_t ldact, int M, int Nh, int K,
                      int gate_first, int activation, int dt, hipStream_t stream);
 
+/* Up to FX_GEMM_MAX_SEGMENTS products that share op(A), as one launch:
+ *   D[i] (M, N[i]) = alpha * op(A) * op(B[i]) + beta * C[i],   i = 0 .. nseg-1.
+ * Replaces back-to-back dispatcher calls whose outputs are each too small to fill the GPU: the key
+ * and value projections of flextrain/nn/blocks/attention.py:424-463 and their weight gradients
+ * (attention.py:712-775).  trans_a / trans_b as in dispatch_matmul (1 = the operand is stored
+ * transposed, i.e. column-major); every B[i] has the same form and its own ldb[i]; C and D are
+ * row-major with strides ldc[i] / ldd[i], C (or ldc) may be NULL when beta is 0.  bf16 or fp16,
+ * outputs of the input type; operands 16-byte aligned with contiguous axes and leading dimensions
+ * multiples of 8 (anything else is an error: the caller falls back to separate calls). */
+#define FX_GEMM_MAX_SEGMENTS 4
+int fx_gemm_segments(const void* A, int64_t lda, int trans_a, int nseg, const void* const* B,
+                     const int64_t* ldb, int trans_b, const void* const* C, const int64_t* ldc,
+                     void* const* D, const int64_t* ldd, int M, const int* N, int K, float alpha,
+                     float beta, int dt, hipStream_t stream);
+
 /* ---- GEMM dispatcher (verbatim ABI of the reference helper) --------------- */
 
 /* helpers/matmul_dispatcher/src/dispatch.h:12-35.  D = alpha*op(A)*op(B) + beta*C,

@@ -128,3 +128,72 @@ def test_long_k_few_tiles_splits_along_k(dev, M, N, K, ta, tb):
     D2 = torch.empty_like(D)
     disp.matmul_fast(s, Ad, Bd, D=D2)
     _check(D2, _ref(A, B), torch.bfloat16)
+
+
+# ---------------------------------------------------------------- products that share A, one launch
+@pytest.mark.parametrize("M,K,Ns", [(512, 1024, (256, 256)),            # 128 x 128 tiles
+                                    (4096, 512, (1024, 1024)),          # 256 x 256 tiles
+                                    (696, 328, (136, 1000, 8)),         # ragged everywhere, three segments
+                                    (4104, 192, (520, 264, 256, 1032))])  # four segments, large tile
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_shared_a_products_in_one_launch(dev, M, K, Ns, ta, tb):
+    g = gen(M + K + sum(Ns) + 2 * ta + tb)
+    A = randn(g, M, K, std=0.5)
+    Bs = [randn(g, K, n, std=0.5) for n in Ns]
+    Cs = [randn(g, M, n) for n in Ns]
+    Ad = A.t().contiguous().to(dev).t() if ta else A.to(dev)
+    Bd = [b.t().contiguous().to(dev).t() if tb else b.to(dev) for b in Bs]
+    disp = CublasLtDispatcher()
+    s = torch.cuda.current_stream().cuda_stream
+    assert disp._segments_ok(Ad, Bd, [torch.empty(M, n, dtype=torch.bfloat16, device=dev) for n in Ns], None)
+    # beta = 0 into fresh outputs
+    Ds = [torch.full((M, n), float("nan"), dtype=torch.bfloat16, device=dev) for n in Ns]
+    disp.matmul_shared_a(s, Ad, Bd, Ds)
+    for i, n in enumerate(Ns):
+        _check(Ds[i], _ref(A, Bs[i]), torch.bfloat16)
+        # the same tile kernel and K order as a call of its own, when that call takes no K splits
+        alone = disp.matmul(s, Ad, Bd[i])
+        _check(Ds[i], alone.float().cpu(), torch.bfloat16)
+    # accumulate in place: D = 0.5 * A B + 2 C with C is D
+    Dd = [c.to(dev) for c in Cs]
+    disp.matmul_shared_a(s, Ad, Bd, Dd, Cs=Dd, alpha=0.5, beta=2.0)
+    for i in range(len(Ns)):
+        _check(Dd[i], _ref(A, Bs[i], Cs[i], 0.5, 2.0), torch.bfloat16)
+
+
+def test_shared_a_outputs_inside_wider_buffers_and_fp16(dev):
+    g = gen(77)
+    M, K, Ns = 384, 256, (128, 384)
+    A = randn(g, M, K, dtype=torch.float16, std=0.5)
+    Bs = [randn(g, K, n, dtype=torch.float16, std=0.5) for n in Ns]
+    wide = torch.full((M, 1024), 7.0, dtype=torch.float16, device=dev)
+    Ds = [wide[:, 8:8 + Ns[0]], wide[:, 256:256 + Ns[1]]]        # row stride 1024, the first 16-byte aligned only
+    disp = CublasLtDispatcher()
+    disp.matmul_shared_a(torch.cuda.current_stream().cuda_stream, A.to(dev), [b.to(dev) for b in Bs], Ds)
+    for i in range(2):
+        _check(Ds[i], _ref(A, Bs[i]), torch.float16)
+    assert torch.all(wide[:, :8] == 7.0) and torch.all(wide[:, 8 + Ns[0]:256] == 7.0) and torch.all(wide[:, 256 + Ns[1]:] == 7.0)
+
+
+def test_shared_a_falls_back_to_separate_calls(dev):
+    """Operands the one-launch form does not take (fp32 outputs, mixed forms of B, odd sizes) give
+    the same results through one dispatcher call per product."""
+    g = gen(78)
+    M, K = 130, 264
+    A = randn(g, M, K, std=0.5)
+    B0, B1 = randn(g, K, 72, std=0.5), randn(g, K, 200, std=0.5)
+    disp = CublasLtDispatcher()
+    s = torch.cuda.current_stream().cuda_stream
+    Ad = A.to(dev)
+    mixed = [B0.to(dev), B1.t().contiguous().to(dev).t()]
+    Ds = [torch.empty(M, 72, dtype=torch.bfloat16, device=dev), torch.empty(M, 200, dtype=torch.bfloat16, device=dev)]
+    assert not disp._segments_ok(Ad, mixed, Ds, None)
+    disp.matmul_shared_a(s, Ad, mixed, Ds)
+    _check(Ds[0], _ref(A, B0), torch.bfloat16)
+    _check(Ds[1], _ref(A, B1), torch.bfloat16)
+    D32 = [torch.empty(M, 72, dtype=torch.float32, device=dev), torch.empty(M, 200, dtype=torch.float32, device=dev)]
+    assert not disp._segments_ok(Ad, [B0.to(dev), B1.to(dev)], D32, None)
+    disp.matmul_shared_a(s, Ad, [B0.to(dev), B1.to(dev)], D32)
+    _check(D32[0], _ref(A, B0), torch.float32)
+    with pytest.raises(ValueError):
+        disp.matmul_shared_a(s, Ad, mixed, Ds[:1])
