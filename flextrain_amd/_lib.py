@@ -88,6 +88,9 @@ _SIGNATURES = {
     "fx_gemm_segments": (c_int, [c_void_p, c_int64, c_int, c_int, POINTER(c_void_p), POINTER(c_int64), c_int,
                                  POINTER(c_void_p), POINTER(c_int64), POINTER(c_void_p), POINTER(c_int64), c_int,
                                  POINTER(c_int), c_int, c_float, c_float, c_int, c_void_p]),
+    "fx_gemm_ksum": (c_int, [c_int, POINTER(c_void_p), POINTER(c_int64), c_int, POINTER(c_void_p), POINTER(c_int64),
+                             c_int, POINTER(c_int), c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_float,
+                             c_float, c_int, c_int, c_void_p]),
     "fx_copy_fields": (c_int, [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
     "create_dispatcher": (c_void_p, [c_int, c_int]),
     "destroy_dispatcher": (None, [c_void_p]),

@@ -80,6 +80,17 @@ class GQAAttentionProjections:
             self._mm(A, B, Ds[i], C=None if Cs is None else Cs[i], beta=beta)
         return Ds
 
+    def _mm_sum(self, As, Bs, D):
+        """``D = sum_i As[i] @ Bs[i]``: one launch with a single rounding where the dispatcher offers
+        it, else the reference's chain of accumulating calls (attention.py:760-775)."""
+        fused = getattr(self.dispatcher, "matmul_sum", None)
+        if fused is not None:
+            return fused(_stream_ptr(As[0]), As, Bs, D=D)
+        self._mm(As[0], Bs[0], D)
+        for A, B in zip(As[1:], Bs[1:]):
+            self._mm(A, B, D, C=D, beta=1.0)
+        return D
+
     def _rope_freqs(self, device) -> torch.Tensor:
         """inv_freq of the configured RoPE, built once (attention.py:373-390)."""
         if self._inv_freq is None or self._inv_freq.device != device:
@@ -177,9 +188,7 @@ class GQAAttentionProjections:
             grads["g_b_k"].add_(dk2d.sum(dim=0))
             grads["g_b_v"].add_(dv2d.sum(dim=0))
         dx = torch.empty((T, cfg.d_model), dtype=dq2d.dtype, device=dq.device)
-        self._mm(dq2d, weights["w_q"].T, dx)
-        self._mm(dk2d, weights["w_k"].T, dx, C=dx, beta=1.0)
-        self._mm(dv2d, weights["w_v"].T, dx, C=dx, beta=1.0)
+        self._mm_sum([dq2d, dk2d, dv2d], [weights["w_q"].T, weights["w_k"].T, weights["w_v"].T], dx)
         slot.aux["bwd_dq"] = dq2d
         slot.aux["bwd_local_dk"] = dk2d
         slot.aux["bwd_local_dv"] = dv2d

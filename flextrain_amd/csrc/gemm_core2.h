@@ -468,7 +468,9 @@ constexpr size_t gemm2_lds_bytes() {
 // K loop of one workgroup tile: leaves the fp32 accumulators of this wave's sub-tile in `acc`
 // (transposed MFMA layout, see epilogue_tile).  B_DUAL: the B tile's second half comes from a
 // second matrix (OperandView::half); K must then be a multiple of 64.
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_MN, bool B_MN, bool B_DUAL = false>
+// ZERO = false: `acc` already holds partial sums and is added to (a product summed over several
+// operand pairs, one call per pair; the call ends with a barrier, so the next may start at once).
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_MN, bool B_MN, bool B_DUAL = false, bool ZERO = true>
 FX_DEV void gemm_mainloop2(const OperandView<T>& A, const OperandView<T>& B, int K, T* smem,
                            f32x16_t (&acc)[BM / WAVES_M / 32][BN / WAVES_N / 32]) {
     constexpr int NW = WAVES_M * WAVES_N, NT = NW * 64;
@@ -480,12 +482,14 @@ FX_DEV void gemm_mainloop2(const OperandView<T>& A, const OperandView<T>& B, int
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: LDS addresses of the loads stay scalar
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
 
+    if (ZERO) {
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
+            for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+    }
 
     const int nfull = K / GEMM_BK;  // K-steps that need no zero fill
     static_assert(GEMM_BK == 64, "the pipeline below is written out for four sub-steps per K-step");

@@ -108,8 +108,12 @@ class SwiGLUFFN:
         else:
             self._mm(fwd_act.T, dy_resid, grads["g_2"], C=grads["g_2"], beta=1.0)
         dx_ffn_norm_up = torch.empty_like(dy_resid)
-        self._mm(dx1_up, weights["w_1"].T, dx_ffn_norm_up)
-        self._mm(dx3_up, weights["w_3"].T, dx_ffn_norm_up, C=dx_ffn_norm_up, beta=1.0)
+        fused = getattr(self.dispatcher, "matmul_sum", None)
+        if fused is not None:    # both products in one launch, summed in fp32 and rounded once
+            fused(_stream_ptr(dx1_up), [dx1_up, dx3_up], [weights["w_1"].T, weights["w_3"].T], D=dx_ffn_norm_up)
+        else:
+            self._mm(dx1_up, weights["w_1"].T, dx_ffn_norm_up)
+            self._mm(dx3_up, weights["w_3"].T, dx_ffn_norm_up, C=dx_ffn_norm_up, beta=1.0)
         slot.aux["bwd_dx1_up"] = dx1_up
         slot.aux["bwd_dx3_up"] = dx3_up
         return dx_ffn_norm_up

@@ -209,6 +209,72 @@ class CublasLtDispatcher:
                     return False
         return True
 
+    def matmul_sum(self, stream_ptr, As, Bs, C=None, D=None, alpha=1.0, beta=0.0):
+        """``D = alpha * sum_i As[i] @ Bs[i] + beta * C`` for up to four products in ONE launch when
+        the operands allow it (bf16 / fp16; every ``A`` in one form and every ``B`` in one form;
+        16-byte aligned with multiples of 8 on K, the contiguous axes and the leading dimensions):
+        the sum is formed in fp32 and rounded once.  Otherwise one :meth:`matmul` per product,
+        accumulating through ``D`` (rounded after each, as the reference's chains of ``beta = 1``
+        calls are: attention.py:712-775, ffn_dense.py:193-235)."""
+        n = len(As)
+        if n == 0 or len(Bs) != n:
+            raise ValueError("matmul_sum: As and Bs must be non-empty and of the same length")
+        M, N = As[0].shape[0], Bs[0].shape[1]
+        if D is None:
+            D = torch.empty((M, N), dtype=As[0].dtype, device=As[0].device)
+        if self._ksum_ok(As, Bs, C, D):
+            la, lb = [_get_layout(a) for a in As], [_get_layout(b) for b in Bs]
+            vp, i64 = ctypes.c_void_p * n, ctypes.c_int64 * n
+            ks = (ctypes.c_int * n)(*[a.shape[1] for a in As])
+            use_c = C is not None and beta != 0.0
+            rc = self._lib.fx_gemm_ksum(n, vp(*[l[0] for l in la]), i64(*[l[1] for l in la]), la[0][2],
+                                        vp(*[l[0] for l in lb]), i64(*[l[1] for l in lb]), lb[0][2], ks,
+                                        C.data_ptr() if use_c else None, C.stride(0) if use_c else 0, D.data_ptr(),
+                                        D.stride(0), M, N, alpha, beta if use_c else 0.0,
+                                        _dtype_to_enum[As[0].dtype], _dtype_to_enum[D.dtype], stream_ptr)
+            if rc != 0:
+                raise RuntimeError("fx_gemm_ksum failed")
+            return D
+        self.matmul(stream_ptr, As[0], Bs[0], C=C, D=D, alpha=alpha, beta=beta)
+        for i in range(1, n):
+            self.matmul(stream_ptr, As[i], Bs[i], C=D, D=D, alpha=alpha, beta=1.0)
+        return D
+
+    @staticmethod
+    def _ksum_ok(As, Bs, C, D):
+        n = len(As)
+        if not 2 <= n <= 4:
+            return False
+        dt = As[0].dtype
+        if dt not in (torch.bfloat16, torch.float16) or As[0].dim() != 2 or Bs[0].dim() != 2:
+            return False
+        M, N = As[0].shape[0], Bs[0].shape[1]
+        if M == 0 or N == 0:
+            return False
+        if D.dim() != 2 or D.shape != (M, N) or D.stride(1) != 1 or not (D.dtype == dt or (dt == torch.bfloat16 and D.dtype == torch.float32)):
+            return False
+        if C is not None and (C.dim() != 2 or C.shape != (M, N) or C.stride(1) != 1 or C.dtype != D.dtype):
+            return False
+
+        def form(t):     # 0 row-major, 1 column-major, None unsupported
+            if t.dim() != 2 or t.dtype != dt or t.data_ptr() % 16:
+                return None
+            sr, sc = t.stride()
+            if sc == 1 and sr % 8 == 0 and sr < (1 << 23) and t.shape[1] % 8 == 0:
+                return 0
+            if sr == 1 and sc % 8 == 0 and sc < (1 << 23) and t.shape[0] % 8 == 0:
+                return 1
+            return None
+
+        fa, fb = form(As[0]), form(Bs[0])
+        if fa is None or fb is None:
+            return False
+        for a, b in zip(As, Bs):
+            K = a.shape[1]
+            if a.shape[0] != M or b.shape != (K, N) or K == 0 or K % 8 or form(a) != fa or form(b) != fb:
+                return False
+        return True
+
     def matmul_fast(self, stream_ptr, A, B, C=None, D=None, alpha=1.0, beta=0.0):
         """Hot-path variant: no validation, no allocation (``D`` required), no
         wrapper timing.  Bit-identical results to :meth:`matmul`."""

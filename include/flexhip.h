@@ -286,6 +286,19 @@ int fx_gemm_segments(const void* A, int64_t lda, int trans_a, int nseg, const vo
                      void* const* D, const int64_t* ldd, int M, const int* N, int K, float alpha,
                      float beta, int dt, hipStream_t stream);
 
+/* A sum of up to FX_GEMM_MAX_SEGMENTS products into one output, as one launch:
+ *   D (M, N) = alpha * sum_i op(A[i]) * op(B[i]) + beta * C,   op(A[i]): M x K[i], op(B[i]): K[i] x N.
+ * Replaces chains of dispatcher calls with beta = 1 into the same output: dq Wq^T + dk Wk^T + dv Wv^T
+ * of flextrain/nn/blocks/attention.py:712-775 and dx1 W1^T + dx3 W3^T of
+ * flextrain/nn/blocks/ffn_dense.py:193-235.  The sum is formed in fp32 and rounded once.  trans_a /
+ * trans_b as in dispatch_matmul, shared by all products; lda[i] / ldb[i] per product.  bf16 or fp16
+ * inputs, output of the input type or fp32 (bf16 inputs); operands 16-byte aligned, K[i],
+ * contiguous axes and leading dimensions multiples of 8 (anything else is an error: the caller
+ * falls back to separate calls). */
+int fx_gemm_ksum(int nseg, const void* const* A, const int64_t* lda, int trans_a, const void* const* B,
+                 const int64_t* ldb, int trans_b, const int* K, const void* C, int64_t ldc, void* D,
+                 int64_t ldd, int M, int N, float alpha, float beta, int dt, int d_dt, hipStream_t stream);
+
 /* ---- GEMM dispatcher (verbatim ABI of the reference helper) --------------- */
 
 /* helpers/matmul_dispatcher/src/dispatch.h:12-35.  D = alpha*op(A)*op(B) + beta*C,

@@ -197,3 +197,76 @@ def test_shared_a_falls_back_to_separate_calls(dev):
     _check(D32[0], _ref(A, B0), torch.float32)
     with pytest.raises(ValueError):
         disp.matmul_shared_a(s, Ad, mixed, Ds[:1])
+
+
+# ---------------------------------------------------------------- a sum of products, one launch
+def _ref_sum(As, Bs, C=None, alpha=1.0, beta=0.0):
+    r = sum(a.float() @ b.float() for a, b in zip(As, Bs)) * alpha
+    if C is not None:
+        r = r + beta * C.float()
+    return r
+
+
+@pytest.mark.parametrize("M,N,Ks", [(512, 384, (256, 64)),               # 128 x 128 tiles
+                                    (4096, 4096, (512, 128, 128)),        # 256 x 256 tiles, short second and third products
+                                    (696, 1000, (200, 72, 8)),            # ragged everywhere, K tails
+                                    (3080, 4104, (64, 192, 136, 320))])   # four products
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_sum_of_products_in_one_launch(dev, M, N, Ks, ta, tb):
+    g = gen(M + N + sum(Ks) + 2 * ta + tb)
+    As = [randn(g, M, k, std=0.5) for k in Ks]
+    Bs = [randn(g, k, N, std=0.5) for k in Ks]
+    C = randn(g, M, N)
+    Ad = [a.t().contiguous().to(dev).t() if ta else a.to(dev) for a in As]
+    Bd = [b.t().contiguous().to(dev).t() if tb else b.to(dev) for b in Bs]
+    disp = CublasLtDispatcher()
+    s = torch.cuda.current_stream().cuda_stream
+    D = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=dev)
+    assert disp._ksum_ok(Ad, Bd, None, D)
+    disp.matmul_sum(s, Ad, Bd, D=D)
+    _check(D, _ref_sum(As, Bs), torch.bfloat16)
+    # against the chain of accumulating calls it replaces (rounded after every product)
+    chain = disp.matmul(s, Ad[0], Bd[0])
+    for a, b in zip(Ad[1:], Bd[1:]):
+        disp.matmul(s, a, b, C=chain, D=chain, beta=1.0)
+    want = _ref_sum(As, Bs)
+    err_fused = (D.float().cpu() - want).abs().mean().item()
+    err_chain = (chain.float().cpu() - want).abs().mean().item()
+    assert err_fused <= err_chain * 1.02 + 1e-6     # one rounding instead of one per product
+    # alpha, beta and C is D; fp32 output
+    Dc = C.to(dev)
+    disp.matmul_sum(s, Ad, Bd, C=Dc, D=Dc, alpha=0.5, beta=2.0)
+    _check(Dc, _ref_sum(As, Bs, C, 0.5, 2.0), torch.bfloat16)
+    D32 = torch.empty(M, N, dtype=torch.float32, device=dev)
+    assert disp._ksum_ok(Ad, Bd, None, D32)
+    disp.matmul_sum(s, Ad, Bd, D=D32)
+    _check(D32, _ref_sum(As, Bs), torch.float32)
+
+
+def _check_chain(D, want):
+    """A chain of accumulating bf16 calls rounds after every product: twice the single-rounding bound."""
+    got = D.float().cpu()
+    scale = max(want.abs().max().item(), 1.0)
+    assert (got - want).abs().max().item() <= 5e-2 * scale
+    assert ((got - want).abs() <= 2e-2 * want.abs() + 1e-3 * scale).float().mean().item() > 0.999
+
+
+def test_sum_of_products_falls_back_to_a_chain(dev):
+    g = gen(91)
+    M, N = 130, 72
+    As = [randn(g, M, 264, std=0.5), randn(g, M, 100, std=0.5)]     # K = 100 is not a multiple of 8
+    Bs = [randn(g, 264, N, std=0.5), randn(g, 100, N, std=0.5)]
+    disp = CublasLtDispatcher()
+    s = torch.cuda.current_stream().cuda_stream
+    Ad, Bd = [a.to(dev) for a in As], [b.to(dev) for b in Bs]
+    D = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    assert not disp._ksum_ok(Ad, Bd, None, D)
+    out = disp.matmul_sum(s, Ad, Bd)
+    _check_chain(out, _ref_sum(As, Bs))
+    C = randn(g, M, N)
+    Dc = C.to(dev)
+    disp.matmul_sum(s, Ad, Bd, C=Dc, D=Dc, alpha=2.0, beta=0.5)
+    # the chain applies alpha to every product and beta to C once
+    _check_chain(Dc, _ref_sum(As, Bs, C, 2.0, 0.5))
+    with pytest.raises(ValueError):
+        disp.matmul_sum(s, Ad, Bd[:1])
