@@ -120,13 +120,22 @@ class SwiGLUFFN:
 
     def bwd_accumulate_w1_w3_grads(self, ffn_norm_output, grads, slot, *, skip_grads: frozenset = frozenset(),
                                    capture_xy: dict | None = None) -> None:
+        todo = []
         for name, dy_key in (("g_1", "bwd_dx1_up"), ("g_3", "bwd_dx3_up")):
             dy = slot.aux[dy_key]
             if name in skip_grads:
                 if capture_xy is not None:
                     capture_xy[name] = (ffn_norm_output, dy)
             else:
-                self._mm(ffn_norm_output.T, dy, grads[name], C=grads[name], beta=1.0)
+                todo.append((name, dy))
+        shared = getattr(self.dispatcher, "matmul_shared_a", None)
+        if len(todo) == 2 and shared is not None:
+            # one grid for both: 2 x 3.5 rounds of workgroups (Llama-3.1-8B shapes) become 7 full ones
+            g = [grads[n] for n, _ in todo]
+            shared(_stream_ptr(ffn_norm_output), ffn_norm_output.T, [dy for _, dy in todo], g, Cs=g, alpha=1.0, beta=1.0)
+            todo = []
+        for name, dy in todo:
+            self._mm(ffn_norm_output.T, dy, grads[name], C=grads[name], beta=1.0)
         del slot.aux["bwd_dx1_up"]
         del slot.aux["bwd_dx3_up"]
 
