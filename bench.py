@@ -86,18 +86,35 @@ def _op_entry(name, work, unit, ms):
             "unit": unit, "frac": round(ach / peak, 4)}
 
 
-def _time_launches(torch, stream, fns, warmup=5, reps=20):
+def _time_launches(torch, stream, fns, warmup=5, reps=20, settle_ms=40.0, window_ms=20.0):
     """Mean milliseconds per launch; ``fns`` is a list of equivalent closures over
     distinct buffer sets, called round-robin so small working sets cannot sit in
-    the 256 MB last-level cache between launches."""
+    the 256 MB last-level cache between launches.
+
+    Coming from idle, the GPU runs MFMA-heavy kernels at boost clocks for the first few
+    milliseconds, then drops below its sustained clocks and recovers over roughly 25 ms (one
+    8192 x 4096 x 4096 GEMM: 222 us, then up to 281 us, then 214 us from the hundredth call on).
+    The timed window therefore starts after at least ``settle_ms`` of the same work and covers at
+    least ``window_ms``: the figure is the sustained one."""
+    n = len(fns)
     with torch.cuda.stream(stream):
-        for i in range(warmup):
-            fns[i % len(fns)]()
         a = torch.cuda.Event(enable_timing=True)
         b = torch.cuda.Event(enable_timing=True)
         a.record(stream)
+        for i in range(max(warmup, 1)):
+            fns[i % n]()
+        b.record(stream)
+        torch.cuda.synchronize()
+        est = max(a.elapsed_time(b) / max(warmup, 1), 1e-3)
+        done = max(warmup, 1)
+        extra = min(2000, int(max(0.0, settle_ms - est * done) / est))
+        for i in range(extra):
+            fns[(done + i) % n]()
+        done += extra
+        reps = max(reps, min(2000, int(window_ms / est) + 1))
+        a.record(stream)
         for i in range(reps):
-            fns[i % len(fns)]()
+            fns[(done + i) % n]()
         b.record(stream)
         torch.cuda.synchronize()
     return a.elapsed_time(b) / reps
