@@ -270,3 +270,41 @@ def test_sum_of_products_falls_back_to_a_chain(dev):
     _check_chain(Dc, _ref_sum(As, Bs, C, 2.0, 0.5))
     with pytest.raises(ValueError):
         disp.matmul_sum(s, Ad, Bd[:1])
+
+
+def test_fused_entry_points_reject_what_they_cannot_take(dev):
+    """Through the C ABI directly: a non-zero return and no launch for counts out of range,
+    misaligned operands, sizes off the 8-element grid and unsupported dtypes."""
+    import ctypes
+
+    from flextrain_amd._lib import lib
+
+    L = lib()
+    s = torch.cuda.current_stream().cuda_stream
+    A = torch.zeros(64, 72, dtype=torch.bfloat16, device=dev)
+    B = torch.zeros(72, 64, dtype=torch.bfloat16, device=dev)
+    D = torch.full((64, 64), 3.0, dtype=torch.bfloat16, device=dev)
+    vp, i64, ci = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+
+    def segments(nseg, a=A, b=B, ldb=64, n=64, dt=2):
+        m = max(nseg, 1)
+        return L.fx_gemm_segments(a.data_ptr(), 72, 0, nseg, (vp * m)(*[b.data_ptr()] * m), (i64 * m)(*[ldb] * m), 0, None, None,
+                                  (vp * m)(*[D.data_ptr()] * m), (i64 * m)(*[64] * m), 64, (ci * m)(*[n] * m), 72, 1.0, 0.0, dt, s)
+
+    assert segments(2) == 0
+    assert segments(0) != 0 and segments(5) != 0
+    assert segments(2, b=B.view(-1)[4:4 + 64 * 64].view(64, 64)) != 0      # B 8 bytes off the 16-byte grid
+    assert segments(2, n=60) != 0                                          # columns of a (K, N) operand not a multiple of 8
+    assert segments(2, dt=0) != 0                                          # fp32 inputs
+
+    def ksum(nseg, k=72, d_dt=2, dt=2):
+        m = max(nseg, 1)
+        return L.fx_gemm_ksum(nseg, (vp * m)(*[A.data_ptr()] * m), (i64 * m)(*[72] * m), 0, (vp * m)(*[B.data_ptr()] * m),
+                              (i64 * m)(*[64] * m), 0, (ci * m)(*[k] * m), None, 0, D.data_ptr(), 64, 64, 64, 1.0, 0.0, dt, d_dt, s)
+
+    assert ksum(2) == 0
+    assert ksum(0) != 0 and ksum(5) != 0
+    assert ksum(2, k=68) != 0 and ksum(2, k=0) != 0
+    assert ksum(2, d_dt=1) != 0 and ksum(2, dt=1, d_dt=0) != 0            # bf16 -> fp16, fp16 -> fp32
+    torch.cuda.synchronize()
+    assert torch.all(D == 0)     # the accepted calls wrote zeros (A, B are zero); the rejected ones nothing
