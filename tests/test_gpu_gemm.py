@@ -308,3 +308,16 @@ def test_fused_entry_points_reject_what_they_cannot_take(dev):
     assert ksum(2, d_dt=1) != 0 and ksum(2, dt=1, d_dt=0) != 0            # bf16 -> fp16, fp16 -> fp32
     torch.cuda.synchronize()
     assert torch.all(D == 0)     # the accepted calls wrote zeros (A, B are zero); the rejected ones nothing
+
+
+def test_sum_of_products_fp16(dev):
+    g = gen(93)
+    M, N, Ks = 520, 392, (128, 72)
+    As = [randn(g, M, k, dtype=torch.float16, std=0.5) for k in Ks]
+    Bs = [randn(g, k, N, dtype=torch.float16, std=0.5) for k in Ks]
+    disp = CublasLtDispatcher()
+    Ad, Bd = [a.to(dev) for a in As], [b.t().contiguous().to(dev).t() for b in Bs]
+    D = torch.empty(M, N, dtype=torch.float16, device=dev)
+    assert disp._ksum_ok(Ad, Bd, None, D)
+    disp.matmul_sum(torch.cuda.current_stream().cuda_stream, Ad, Bd, D=D)
+    _check(D, _ref_sum(As, Bs), torch.float16)
