@@ -177,3 +177,47 @@ def test_skip_grads_hands_back_operands(dev):
         GQAAttentionProjections(GQAProjectionConfig(d_model=64, n_heads=4, n_kv_heads=2, head_dim=16, qk_norm=True)).bwd_qkv(
             randn(g, T, 4, 16).to(dev), randn(g, T, 2, 16).to(dev), randn(g, T, 2, 16).to(dev), pos,
             dict(W, w_q_norm=torch.ones(16, device=dev), w_k_norm=torch.ones(16, device=dev)), G, slot)
+
+
+class _MatmulOnly:
+    """A dispatcher with the reference's surface only (``matmul``)."""
+
+    def __init__(self):
+        from flextrain_amd.matmul_dispatcher import CublasLtDispatcher
+        self._d = CublasLtDispatcher()
+        self.calls = 0
+
+    def matmul(self, stream_ptr, A, B, C=None, D=None, alpha=1.0, beta=0.0):
+        self.calls += 1
+        return self._d.matmul(stream_ptr, A, B, C=C, D=D, alpha=alpha, beta=beta)
+
+
+def test_block_over_a_dispatcher_without_fused_launches(dev):
+    """The one-launch forms (key / value projections and weight gradients, the summed input gradient) are
+    optional: over a dispatcher that only has ``matmul`` the block issues the reference's 12 calls and
+    gives the same results within rounding."""
+    g = gen(23)
+    T, d, H, Hkv, D = 256, 256, 8, 2, 64
+    cfg = GQAProjectionConfig(d_model=d, n_heads=H, n_kv_heads=Hkv, head_dim=D, rope_theta=10000.0)
+    w, _ = _setup(g, cfg, T, bf)
+    x, resid, dy = randn(g, T, d), randn(g, T, d), randn(g, T, d)
+    attn = randn(g, T, H, D)
+    dq, dk, dv = randn(g, T, H, D), randn(g, T, Hkv, D), randn(g, T, Hkv, D)
+    pos = torch.arange(T, dtype=torch.int32).view(T, 1)
+    results = []
+    for disp in (None, _MatmulOnly()):
+        blk = GQAAttentionProjections(cfg, dispatcher=disp)
+        W = {k: v.to(dev) for k, v in w.items()}
+        G = {"g_" + k: torch.zeros_like(W["w_" + k]) for k in "qkvo"}
+        slot = _slot(cfg, T, dev)
+        blk.fwd_qkv(x.to(dev), pos.to(dev), W, slot)
+        slot.attn_result.copy_(attn.to(dev))
+        out = blk.fwd_o(resid.to(dev), W, slot)
+        dattn = blk.bwd_o(dy.to(dev), W, G, slot)
+        dx = blk.bwd_qkv(dq.to(dev), dk.to(dev), dv.to(dev), pos.to(dev), W, G, slot, attn_norm_output=x.to(dev))
+        blk.bwd_accumulate_qkv_grads(x.to(dev), G, slot)
+        results.append((slot.xq, slot.xk, slot.xv, out, dattn, dx, G["g_q"], G["g_k"], G["g_v"], G["g_o"]))
+        if disp is not None:
+            assert disp.calls == 12
+    for name, a, b in zip(("xq", "xk", "xv", "xo", "dattn", "dx", "g_q", "g_k", "g_v", "g_o"), *results):
+        _close(b.reshape(a.shape), a.float().cpu(), name)

@@ -69,3 +69,40 @@ def test_skip_grads_hands_back_operands(dev):
     assert set(cap) == {"g_1", "g_2", "g_3"} and not any(v.any() for v in G.values())
     act, dyc = cap["g_2"]
     assert act.shape == (T, f) and torch.equal(dyc, dy) and cap["g_1"][0] is h
+
+
+class _MatmulOnly:
+    """A dispatcher with the reference's surface only (``matmul``): the blocks must then issue the
+    reference's chains of separate calls."""
+
+    def __init__(self):
+        from flextrain_amd.matmul_dispatcher import CublasLtDispatcher
+        self._d = CublasLtDispatcher()
+        self.calls = 0
+
+    def matmul(self, stream_ptr, A, B, C=None, D=None, alpha=1.0, beta=0.0):
+        self.calls += 1
+        return self._d.matmul(stream_ptr, A, B, C=C, D=D, alpha=alpha, beta=beta)
+
+
+def test_block_over_a_dispatcher_without_fused_launches(dev):
+    g = gen(11)
+    T, d, f = 256, 128, 328
+    bf = torch.bfloat16
+    h, resid, dy = randn(g, T, d), randn(g, T, d), randn(g, T, d)
+    w = {"w_1": randn(g, d, f, std=d ** -0.5), "w_3": randn(g, d, f, std=d ** -0.5), "w_2": randn(g, f, d, std=f ** -0.5)}
+    results = []
+    for disp in (None, _MatmulOnly()):
+        blk = SwiGLUFFN(SwiGLUConfig(d_model=d, expert_dim=f, activation="silu"), dispatcher=disp)
+        W = {k: v.to(dev) for k, v in w.items()}
+        G = {"g_1": torch.zeros(d, f, dtype=bf, device=dev), "g_2": torch.zeros(f, d, dtype=bf, device=dev),
+             "g_3": torch.zeros(d, f, dtype=bf, device=dev)}
+        slot = SimpleNamespace(x1=torch.empty(T, f, dtype=bf, device=dev), x3=torch.empty(T, f, dtype=bf, device=dev), aux={})
+        out = blk.fwd(h.to(dev), W, resid.to(dev), torch.empty(T, d, dtype=bf, device=dev), slot)
+        dx = blk.bwd(dy.to(dev), W, G, slot)
+        blk.bwd_accumulate_w1_w3_grads(h.to(dev), G, slot)
+        results.append((out, dx, G["g_1"], G["g_2"], G["g_3"]))
+        if disp is not None:
+            assert disp.calls >= 7     # down projection; 4 in bwd (the input gradient as a chain of 2); 2 weight gradients
+    for name, a, b in zip(("out", "dx", "g_1", "g_2", "g_3"), *results):
+        _close(b, a.float().cpu(), name)
