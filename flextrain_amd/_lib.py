@@ -100,13 +100,13 @@ _SIGNATURES = {
                                 c_int, c_int, c_float, c_float, c_int, c_int]),
     "fx_host_alloc": (c_int, [c_size_t, POINTER(c_void_p)]),
     "fx_host_free": (c_int, [c_void_p]),
-    "fx_host_register": (c_int, [c_void_p, c_size_t]),
-    "fx_host_unregister": (c_int, [c_void_p]),
+    "fx_stream_ring_create": (c_int, [c_int, POINTER(c_void_p)]),
+    "fx_stream_ring_destroy": (c_int, [c_void_p]),
     "fx_adamw_stream_ws_bytes": (c_size_t, [c_int64, c_int, c_int, c_int, c_int, c_int]),
     "fx_adamw_stream_chunk": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int,
                                       c_int, c_int, c_float, c_float, c_float, c_float, c_float, c_float,
                                       c_float, c_void_p, c_size_t, c_int64, c_int, c_void_p, c_void_p,
-                                      c_void_p]),
+                                      c_void_p, c_void_p]),
     "fx_probe_ws_bytes": (c_size_t, []),
     "fx_probe_mfma_rate": (c_int, [c_int, c_int, c_void_p, c_size_t, POINTER(c_double), c_void_p]),
     "solve_scheduler": (c_double, [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_double, c_int, c_int,

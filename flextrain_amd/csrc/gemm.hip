@@ -174,13 +174,22 @@ static bool mfma_ok(const void* A, const void* B, int M, int N, int K, int64_t l
     return true;
 }
 
+// Everything the choice of kernel depends on.  `facts` holds what is not a shape: whether A and B are
+// 16-byte aligned (the MFMA kernels load 16 bytes per lane straight from the operands, so a view that
+// starts 2 elements into a row must not reuse the entry an aligned call made, and an unaligned first
+// call must not pin the slow kernel on the shape), and whether a C term is read (its dtype only
+// matters then).
 struct ShapeKey {
-    int M, N, K, lda, ldb, ldc, ldd, a_dt, b_dt, c_dt, d_dt, ta, tb;
+    int M, N, K, lda, ldb, ldc, ldd, a_dt, b_dt, c_dt, d_dt, ta, tb, facts;
     bool operator==(const ShapeKey& o) const {
         return M == o.M && N == o.N && K == o.K && lda == o.lda && ldb == o.ldb && ldc == o.ldc && ldd == o.ldd &&
-               a_dt == o.a_dt && b_dt == o.b_dt && c_dt == o.c_dt && d_dt == o.d_dt && ta == o.ta && tb == o.tb;
+               a_dt == o.a_dt && b_dt == o.b_dt && c_dt == o.c_dt && d_dt == o.d_dt && ta == o.ta && tb == o.tb &&
+               facts == o.facts;
     }
 };
+static inline int key_facts(const void* A, const void* B, bool has_c) {
+    return (aligned16(A) ? 1 : 0) | (aligned16(B) ? 2 : 0) | (has_c ? 4 : 0);
+}
 struct ShapeHash {
     size_t operator()(const ShapeKey& k) const {
         size_t h = 1469598103934665603ull;
@@ -254,7 +263,7 @@ extern "C" int dispatch_matmul(DispatchContext* ctx, intptr_t stream_ptr, int M,
 
     ctx->calls++;
     const uint64_t h0 = now_ns();
-    ShapeKey key{M, N, K, lda, ldb, ldc, ldd, a_dt, b_dt, c_dt, d_dt, trans_a, trans_b};
+    ShapeKey key{M, N, K, lda, ldb, ldc, ldd, a_dt, b_dt, c_dt, d_dt, trans_a, trans_b, key_facts(A, B, has_c)};
     const uint64_t h1 = now_ns();
     int cfg;
     auto it = ctx->exact.find(key);
@@ -263,7 +272,7 @@ extern "C" int dispatch_matmul(DispatchContext* ctx, intptr_t stream_ptr, int M,
         ctx->hits++;
     } else {
         const int r = ctx->round_multiple;
-        ShapeKey fk{round_up(M, r), round_up(N, r), round_up(K, r), 0, 0, 0, 0, a_dt, b_dt, c_dt, d_dt, trans_a, trans_b};
+        ShapeKey fk{round_up(M, r), round_up(N, r), round_up(K, r), 0, 0, 0, 0, a_dt, b_dt, c_dt, d_dt, trans_a, trans_b, 0};
         const bool fast = mfma_ok(A, B, M, N, K, lda, ldb, a_dt, b_dt, c_dt, d_dt, trans_a, trans_b, has_c);
         auto fit = ctx->fuzzy.find(fk);
         if (!fast) {

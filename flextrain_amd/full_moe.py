@@ -76,12 +76,13 @@ def dispatch_scatter(x, router_weights, topk_ids, *, num_experts, index_mapping,
     guarantee that the host counts are readable on return; the grouped expert
     path does not need them and passes ``sync=False``."""
     pinned = expert_counts_cpu if (expert_counts_cpu is not None and expert_counts_cpu.is_pinned()) else None
-    indices, _ = flextrain_moe_sort(topk_ids, num_experts=num_experts, indices=index_mapping,
-                                    expert_counts_gpu=expert_counts_gpu, expert_counts_pinned=pinned)
+    indices, counts = flextrain_moe_sort(topk_ids, num_experts=num_experts, indices=index_mapping,
+                                         expert_counts_gpu=expert_counts_gpu, expert_counts_pinned=pinned)
     flextrain_moe_scatter(x, indices, out=scattered_x_out)
     flextrain_moe_scatter_routing_weights(router_weights, indices, out=scattered_router_weights_out)
     if expert_counts_cpu is not None and pinned is None:
-        expert_counts_cpu.copy_(expert_counts_gpu)  # pageable destination: synchronous copy
+        expert_counts_cpu.copy_(counts)  # pageable destination: synchronous copy (counts: the sort's own
+        # result, valid whether or not the caller lent expert_counts_gpu)
     elif sync:
         torch.cuda.current_stream(x.device).synchronize()
     return indices, expert_counts_cpu

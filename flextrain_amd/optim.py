@@ -56,11 +56,46 @@ class AdamW:
         return 0
 
 
+class AdamWStreamWorkspace:
+    """Device staging memory for :func:`flextrain_adamw_step_streamed` together with the
+    per-slot events that order one call after the previous one on the same memory, so
+    calls for successive chunks / layers may follow each other without synchronising."""
+
+    def __init__(self, sub_elems, n_slots, p_dtype, g_dtype, state_dtype, stage_bf16_copy, device):
+        import ctypes
+
+        self.sub_elems, self.n_slots = int(sub_elems), int(n_slots)
+        nbytes = int(lib().fx_adamw_stream_ws_bytes(self.sub_elems, self.n_slots, dtype_enum(p_dtype),
+                                                    dtype_enum(g_dtype), dtype_enum(state_dtype),
+                                                    1 if stage_bf16_copy else 0))
+        self.buffer = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        # the allocating stream may still own the block's previous life: order every stream after it
+        self.alloc_event = torch.cuda.current_stream(device).record_event()
+        handle = ctypes.c_void_p()
+        check(lib().fx_stream_ring_create(self.n_slots, ctypes.byref(handle)), "fx_stream_ring_create")
+        self._ring = handle
+
+    def numel(self) -> int:
+        return self.buffer.numel()
+
+    def data_ptr(self) -> int:
+        return self.buffer.data_ptr()
+
+    def close(self) -> None:
+        if self._ring is not None:
+            lib().fx_stream_ring_destroy(self._ring)
+            self._ring = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
 def adamw_stream_workspace(sub_elems, n_slots, p_dtype, g_dtype, state_dtype, stage_bf16_copy, device):
-    """Device staging buffer for :func:`flextrain_adamw_step_streamed`."""
-    nbytes = int(lib().fx_adamw_stream_ws_bytes(sub_elems, n_slots, dtype_enum(p_dtype), dtype_enum(g_dtype),
-                                                dtype_enum(state_dtype), 1 if stage_bf16_copy else 0))
-    return torch.empty(nbytes, dtype=torch.uint8, device=device)
+    """Device staging workspace for :func:`flextrain_adamw_step_streamed`."""
+    return AdamWStreamWorkspace(sub_elems, n_slots, p_dtype, g_dtype, state_dtype, stage_bf16_copy, device)
 
 
 def flextrain_adamw_step_streamed(params, grads, exp_avgs, exp_avg_sqs, *, streams: StreamBundle, lr=1e-4, beta1=0.9,
@@ -71,7 +106,14 @@ def flextrain_adamw_step_streamed(params, grads, exp_avgs, exp_avg_sqs, *, strea
     ``streams.compute`` and copied back on ``streams.outbound`` with all three
     overlapping.  ``params_bf16_out`` (optional, bf16, pinned host or device) receives the
     updated parameters rounded to bf16.  Enqueues only; the host tensors hold the result
-    after ``streams.outbound.synchronize()``.  Returns 0."""
+    after ``streams.outbound.synchronize()``.  Returns 0.
+
+    ``workspace`` (:func:`adamw_stream_workspace`) may be passed to successive calls
+    without any synchronisation between them: its slot events order each call's copies
+    after the previous call's kernels and copies on the same staging memory.  A raw
+    ``torch.uint8`` tensor is accepted too; its first copies then wait for everything
+    enqueued so far on ``compute`` and ``outbound``.  The caller still orders the three
+    streams after whatever PRODUCED the host tensors (e.g. a gradient offload)."""
     n = params.numel()
     for t, name in ((params, "params"), (grads, "grads"), (exp_avgs, "exp_avgs"), (exp_avg_sqs, "exp_avg_sqs")):
         if t.is_cuda or not t.is_pinned():
@@ -91,20 +133,30 @@ def flextrain_adamw_step_streamed(params, grads, exp_avgs, exp_avg_sqs, *, strea
     if n == 0:
         return 0
     device = streams.compute.device
-    sub_elems = max(8, min(int(sub_elems), (n + 7) // 8 * 8))
     stage = params_bf16_out is not None and not out_on_device
+    ring = None
     if workspace is None:
-        workspace = adamw_stream_workspace(sub_elems, n_slots, params.dtype, grads.dtype, exp_avgs.dtype, stage, device)
+        sub_elems = max(8, min(int(sub_elems), (n + 7) // 8 * 8))
+        workspace = AdamWStreamWorkspace(sub_elems, n_slots, params.dtype, grads.dtype, exp_avgs.dtype, stage, device)
+    if isinstance(workspace, AdamWStreamWorkspace):
+        sub_elems, n_slots, ring, buf = workspace.sub_elems, workspace.n_slots, workspace._ring, workspace.buffer
+        if workspace.alloc_event is not None:
+            for s in (streams.inbound, streams.compute, streams.outbound):
+                s.wait_event(workspace.alloc_event)
+            workspace.alloc_event = None
+    else:
+        sub_elems = max(8, min(int(sub_elems), (n + 7) // 8 * 8))
+        buf = workspace
     step = max(1, step)
     rc = lib().fx_adamw_stream_chunk(
         params.data_ptr(), grads.data_ptr(), exp_avgs.data_ptr(), exp_avg_sqs.data_ptr(),
         params_bf16_out.data_ptr() if params_bf16_out is not None else None, out_on_device, n,
         dtype_enum(params.dtype), dtype_enum(grads.dtype), dtype_enum(exp_avgs.dtype), lr, beta1, beta2, eps,
-        weight_decay, 1.0 - beta1 ** step, 1.0 - beta2 ** step, workspace.data_ptr(), workspace.numel(), sub_elems,
-        n_slots, streams.inbound.cuda_stream, streams.compute.cuda_stream, streams.outbound.cuda_stream)
+        weight_decay, 1.0 - beta1 ** step, 1.0 - beta2 ** step, buf.data_ptr(), buf.numel(), sub_elems,
+        n_slots, streams.inbound.cuda_stream, streams.compute.cuda_stream, streams.outbound.cuda_stream, ring)
     check(rc, "fx_adamw_stream_chunk")
     # the staging buffer must outlive the enqueued work
-    workspace.record_stream(streams.inbound)
-    workspace.record_stream(streams.compute)
-    workspace.record_stream(streams.outbound)
+    buf.record_stream(streams.inbound)
+    buf.record_stream(streams.compute)
+    buf.record_stream(streams.outbound)
     return 0

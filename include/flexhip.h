@@ -330,13 +330,6 @@ int dispatch_matmul(DispatchContext* ctx, intptr_t stream_ptr, int M, int N, int
 int fx_host_alloc(size_t bytes, void** out);
 int fx_host_free(void* ptr);
 
-/* cudaHostRegister / cudaHostUnregister of flextrain/ops/_kernels/_mem_register.py:4-20
- * and flextrain/engine/host_memory.py:76-106.  fx_host_register returns 0 on a fresh
- * registration, 1 when the range was already registered (benign, as the reference
- * treats error 712), -1 on failure; a failure leaves no pending HIP error behind. */
-int fx_host_register(void* ptr, size_t bytes);
-int fx_host_unregister(void* ptr);
-
 /* send_home / fetch_home of one activation slot (flextrain/core/activation_schema.py:483-519; the
  * engine's call sites are flextrain/engine/active_model.py:1184-1199 and :2036-2098): all n
  * fields in one call.  Field i: rows[i] rows of row_bytes[i] bytes, rows dst_pitch[i] /
@@ -362,12 +355,19 @@ size_t fx_adamw_stream_ws_bytes(int64_t sub_elems, int n_slots, int p_dt, int g_
  * `inbound`, kernels on `compute`, copies out on `outbound` (three distinct non-null
  * streams give full overlap).  Enqueues only: the host buffers hold the result once
  * `outbound` (and, for a device-side bf16 copy, `compute`) has drained.  The caller
- * orders the three streams after whatever produced the host buffers. */
+ * orders the three streams after whatever produced the host buffers.
+ * `ring` (fx_stream_ring_create, same n_slots) carries the slots' "free again" events from one
+ * call to the next on the same workspace, so back-to-back calls need no synchronisation between
+ * them and keep overlapping (the layer-after-layer pattern of ActiveModel.step).  With ring =
+ * NULL the first copies-in wait for all work enqueued so far on `compute` and `outbound`. */
+typedef struct FxStreamRing FxStreamRing;
+int fx_stream_ring_create(int n_slots, FxStreamRing** out);
+int fx_stream_ring_destroy(FxStreamRing* ring);
 int fx_adamw_stream_chunk(void* p_host, const void* g_host, void* m_host, void* v_host, void* p_bf16_out,
                           int p_bf16_out_on_device, int64_t n, int p_dt, int g_dt, int state_dt, float lr,
                           float beta1, float beta2, float eps, float weight_decay, float bias_correction1,
                           float bias_correction2, void* ws, size_t ws_bytes, int64_t sub_elems, int n_slots,
-                          hipStream_t inbound, hipStream_t compute, hipStream_t outbound);
+                          hipStream_t inbound, hipStream_t compute, hipStream_t outbound, FxStreamRing* ring);
 
 /* ---- Hardware probe --------------------------------------------------------- */
 

@@ -12,7 +12,10 @@ Pinned by tests/test_oracle_moe.py: stable descending sort for top-k (with
 deliberate ties), stable argsort / bincount and an O(n^2) rank count for the
 sort, indexing identities for scatter/gather, torch.autograd through
 softmax / silu for every backward, and an eager per-expert MLP with autograd
-for the grouped expert block (tests/moe/test_moe_backend_parity.py:45-107).
+for the grouped expert block (tests/moe/test_moe_backend_parity.py:45-107), and -- for
+the composed block ``routed_block_fwd_bwd`` (routing weights, gather with residual,
+router path, load-balance term, ``experts=`` subset) -- fp64 autograd through the whole
+block written as one differentiable expression with the selection held constant.
 """
 from __future__ import annotations
 

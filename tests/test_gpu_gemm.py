@@ -106,6 +106,42 @@ def test_cache_statistics_and_noop(dev):
         tensor_layout(torch.ones(8, 8, 2, device=dev)[:, :, 0])
 
 
+@pytest.mark.parametrize("fast", [False, True])
+@pytest.mark.parametrize("first_aligned", [True, False])
+def test_one_dispatcher_aligned_then_offset_view_then_aligned(dev, fast, first_aligned):
+    """The cached kernel choice must follow operand alignment: a column slice that starts 2 elements
+    (4 bytes) into a row has the same shape and leading dimension as the aligned operand but cannot
+    take the 16-byte loads of the MFMA kernel, and an unaligned first call must not pin the
+    one-element-per-lane kernel on later aligned calls of that shape."""
+    g = gen(91)
+    M, N, K = 384, 512, 256
+    wide = randn(g, M, K + 8, std=0.5)                   # lda = K + 8 for every view below
+    B = randn(g, K, N, std=0.5)
+    wd, Bd = wide.to(dev), B.to(dev)
+    views = {True: (wide[:, :K], wd[:, :K]), False: (wide[:, 2:2 + K], wd[:, 2:2 + K])}
+    assert views[True][1].data_ptr() % 16 == 0 and views[False][1].data_ptr() % 16 == 4
+    disp = CublasLtDispatcher()
+    s = torch.cuda.current_stream().cuda_stream
+    call = disp.matmul_fast if fast else disp.matmul
+    order = [first_aligned, not first_aligned, first_aligned, not first_aligned]
+    outs = []
+    for aligned in order:
+        D = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+        call(s, views[aligned][1], Bd, D=D)
+        _check(D, _ref(views[aligned][0], B), torch.bfloat16)
+        outs.append(D)
+    assert torch.equal(outs[0], outs[2]) and torch.equal(outs[1], outs[3])
+    st = disp.get_stats()
+    # one MFMA tile choice saved (by the aligned call), calls 3 and 4 are exact hits of their own entries
+    assert (st["matmuls_called"], st["algos_saved"], st["algo_hits"]) == (4, 1, 2)
+    # the aligned calls ran the MFMA kernel, the offset ones did not: bf16 accumulation order differs
+    # between the two kernels, but each is deterministic
+    C0 = randn(g, M, N)
+    Dc = C0.to(dev).clone()
+    call(s, views[True][1], Bd, C=Dc, D=Dc, beta=1.0)     # same shape with a C term: a separate entry again
+    _check(Dc, _ref(views[True][0], B, C0, 1.0, 1.0), torch.bfloat16)
+
+
 @pytest.mark.parametrize("M,N,K,ta,tb", [(256, 512, 16384, 0, 0), (300, 520, 8200, 0, 1), (1024, 4096, 32064, 0, 0),
                                          (512, 256, 12288, 1, 0)])
 def test_long_k_few_tiles_splits_along_k(dev, M, N, K, ta, tb):

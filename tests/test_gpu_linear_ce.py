@@ -105,6 +105,22 @@ def test_fused_softmax_ce(dev, T, V, dtype):
     assert torch.equal(xd2.cpu(), x) and torch.equal(out, dz)
 
 
+class _KeepLogits:
+    """A loss object (the head's ``loss_fn=`` hook) that keeps a copy of the bf16 logits the head
+    produced before the wrapped loss turns them into dZ in place, so that the fp32 loss can be
+    checked against ``F.cross_entropy`` of the SAME logits at the fp32 tolerance."""
+
+    def __init__(self, inner):
+        self.inner, self.kept = inner, []
+
+    def compute(self, logits, token_slice, *, loss_scale, per_token_loss_out):
+        self.kept.append(logits.cpu())
+        return self.inner.compute(logits, token_slice, loss_scale=loss_scale, per_token_loss_out=per_token_loss_out)
+
+    def logits(self):
+        return torch.cat(self.kept)
+
+
 def _head_inputs(seed, T, d, V, hf_layout):
     g = gen(seed)
     x = randn(g, T, d)
@@ -130,16 +146,21 @@ def test_lm_head_forward_backward(dev, hf_layout, fused, fuse_chunks):
     g_norm = torch.zeros(d, dtype=torch.float32, device=dev)
     head = LMHead(LMHeadConfig(d_model=d, vocab_size=V, head_chunk_size=chunk, fuse_chunks=fuse_chunks))
     xd = x.to(dev)
+    keep = _KeepLogits(CrossEntropyLoss(fused=fused))
     dx, stats = head.forward_backward(xd, TokenContext(labels=labels.to(dev)), None,
                                       {"w_final_norm": w_norm.to(dev), "w_head_proj": wd},
                                       {"g_head_proj": g_head, "g_final_norm": g_norm}, None, loss_scale=scale,
-                                      loss_fn=CrossEntropyLoss(fused=fused))
+                                      loss_fn=keep)
     assert dx is xd and stats.token_count == T
     if fused:
         close(stats.per_token_loss, ref["per_token_loss"], rtol=1e-2, atol=2e-2, what="per-token loss")
-        # mean loss: fp32, 1e-4 relative once the logits are the same bf16 values; the two sides' logits
-        # differ by GEMM accumulation order, which averages out over tokens
-        close(stats.per_token_loss.sum() * scale, ref["per_token_loss"].sum() * scale, rtol=1e-3, atol=0, what="mean loss")
+        # fp32 loss at rtol 1e-4: against fp32 cross-entropy of the very bf16 logits the head produced
+        # (the oracle's own logits differ from them by GEMM accumulation order, a bf16-sized effect)
+        want = F.cross_entropy(keep.logits().float(), labels, ignore_index=-100, reduction="none")
+        close(stats.per_token_loss, want, rtol=F32_RTOL, atol=1e-5, what="per-token loss from the same logits")
+        close(stats.per_token_loss.sum() * scale, want.sum() * scale, rtol=F32_RTOL, atol=0, what="mean loss")
+        close(stats.per_token_loss.sum() * scale, ref["per_token_loss"].sum() * scale, rtol=1e-3, atol=0,
+              what="mean loss against the oracle's own logits")
     else:
         close(stats.per_token_loss.sum() * scale, ref["per_token_loss"].sum() * scale, rtol=1e-2, atol=0, what="mean loss")
     ign = labels == -100
@@ -187,17 +208,27 @@ def test_full_size_llama_head(dev):
     scale = 1.0 / int((labels != -100).sum())
     wd, ld, wn = w.to(dev), labels.to(dev), w_norm.to(dev)
 
-    def run(fuse):
+    def run(fuse, loss_fn=None):
         xd = x.to(dev)
         gh = torch.zeros(V, d, dtype=torch.float32, device=dev)
         gn = torch.zeros(d, dtype=torch.float32, device=dev)
         head = LMHead(LMHeadConfig(d_model=d, vocab_size=V, head_chunk_size=chunk, fuse_chunks=fuse))
         dx, stats = head.forward_backward(xd, TokenContext(labels=ld), None, {"w_final_norm": wn, "w_head_proj": wd.t()},
-                                          {"g_head_proj": gh.t(), "g_final_norm": gn}, None, loss_scale=scale)
+                                          {"g_head_proj": gh.t(), "g_final_norm": gn}, None, loss_scale=scale,
+                                          loss_fn=loss_fn)
         return dx, stats, gh, gn
 
     dx, stats, gh, gn = run(None)
-    dx1, stats1, gh1, gn1 = run(1)
+    keep = _KeepLogits(CrossEntropyLoss())
+    dx1, stats1, gh1, gn1 = run(1, keep)
+    # fp32 loss at rtol 1e-4, all 8192 tokens: fp32 cross-entropy (library routine, CPU) of the bf16
+    # logits the head itself produced, one micro-chunk at a time
+    want = torch.cat([F.cross_entropy(lg.float(), labels[i * chunk:(i + 1) * chunk], ignore_index=-100,
+                                      reduction="none") for i, lg in enumerate(keep.kept)])
+    keep.kept.clear()
+    close(stats1.per_token_loss, want, rtol=F32_RTOL, atol=1e-5, what="per-token loss from the same logits")
+    close(stats1.per_token_loss.sum() * scale, want.sum() * scale, rtol=F32_RTOL, atol=0, what="mean loss of 8192 tokens")
+    close(stats.per_token_loss.sum() * scale, want.sum() * scale, rtol=F32_RTOL, atol=0, what="mean loss, grouped schedule")
     # schedule independence (accumulation order differs: bf16 dx, fp32 head gradient)
     close(stats.per_token_loss, stats1.per_token_loss, rtol=1e-4, atol=1e-4, what="loss grouped vs per chunk")
     close(dx, dx1, rtol=1e-2, atol=1e-2 * dx1.float().abs().max().item(), what="dx grouped vs per chunk")

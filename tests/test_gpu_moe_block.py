@@ -156,7 +156,8 @@ def _run_block(dev, T, d, E, K, F, seed, lb=0.0, experts=None, init_grads=False)
     logits = slot.x_router.cpu()                         # routing is exact only from identical logits
     ref = o_moe.routed_block_fwd_bwd(x, logits, w_router, w_up, w_down, res, dy, K, load_balance_coef=lb,
                                      tokens_per_step=4 * T if lb else None, experts=experts)
-    return dict(out=out, dx=dx, grads=grads, slot=slot, ref=ref, g0=g0, x=x, w_router=w_router,
+    return dict(out=out, dx=dx, grads=grads, slot=slot, ref=ref, g0=g0, x=x, w_router=w_router, res=res, dy=dy,
+                weights_cpu=dict(w_router=w_router, w_up=w_up, w_down=w_down),
                 host_counts=chunk_extra[backend._CHUNK_EXTRA_HOST_COUNTS][3])
 
 
@@ -183,8 +184,9 @@ def test_block_fwd_bwd(dev, T, d, E, K, F, lb, init):
 
 def test_block_full_size_qwen3_30b_a3b(dev):
     """8192 tokens, hidden 2048, 128 experts, top-8, intermediate 768.  The oracle
-    evaluates 6 of the 128 experts (their row ranges, g_up/g_down slices); routing,
-    permutation and counts are checked for every token."""
+    evaluates 6 of the 128 experts (their row ranges, g_up/g_down slices) and, with all
+    experts, the output and dx of 64 sampled tokens; routing, permutation and counts are
+    checked for every token."""
     picks = (0, 1, 31, 64, 100, 127)
     r = _run_block(dev, 8192, 2048, 128, 8, 768, seed=1004, experts=picks)
     ref, slot = r["ref"], r["slot"]
@@ -197,9 +199,17 @@ def test_block_full_size_qwen3_30b_a3b(dev):
         _close_scaled(slot.x_up[a:b], ref["pre"][a:b], f"x_up rows of expert {e}")
         _close_scaled(r["grads"]["g_up"][e], ref["g_up"][e], f"g_up[{e}]", tol=2e-2)
         _close_scaled(r["grads"]["g_down"][e], ref["g_down"][e], f"g_down[{e}]", tol=2e-2)
-    # tokens whose 8 experts all lie in the evaluated subset: none in general, so check
-    # the output through its invariant instead: out - residual is a convex combination
-    # bounded by the largest expert-output row norm
+    # out and dx at full size: every token's rows are independent of the other tokens' (the grouped
+    # buffers only reorder them; tests/test_oracle_moe.py pins that property of the oracle), so the
+    # oracle runs the whole block, all 128 experts, on a sample of tokens with the GPU's own logits
+    g = gen(77)
+    tok = torch.cat([torch.tensor([0, 1, 4095, 4096, 8190, 8191]), torch.randint(0, 8192, (58,), generator=g)])
+    xs, ws = r["x"], r["weights_cpu"]
+    small = o_moe.routed_block_fwd_bwd(xs[tok], slot.x_router.cpu()[tok], ws["w_router"], ws["w_up"], ws["w_down"],
+                                       r["res"][tok], r["dy"][tok], 8)
+    assert torch.equal(small["ids"], ref["ids"][tok])
+    _close_scaled(r["out"].cpu()[tok], small["out"], "out of 64 sampled tokens")
+    _close_scaled(r["dx"].cpu()[tok], small["dx"], "dx of 64 sampled tokens", tol=2e-2)
     assert torch.isfinite(r["out"].float()).all() and torch.isfinite(r["dx"].float()).all()
     assert int(slot.expert_counts.sum()) == 8192 * 8
 
@@ -222,6 +232,14 @@ def test_recompute_and_phase_ops(dev):
                                            expert_counts_gpu=slot.expert_counts, expert_counts_cpu=host,
                                            scattered_x_out=sx, scattered_router_weights_out=slot.scattered_router_weights)
     assert host2 is host and int(host.sum()) == T * K      # readable on return (sync=True default)
+    # pageable host counts and no device counts buffer lent: the sort's own counts are copied
+    pageable = torch.zeros(E, dtype=torch.int32)
+    sx2 = torch.empty_like(sx)
+    srw2 = torch.empty_like(slot.scattered_router_weights)
+    idx2, host3 = full_moe.dispatch_scatter(x, rw, ids, num_experts=E, index_mapping=None, expert_counts_gpu=None,
+                                            expert_counts_cpu=pageable, scattered_x_out=sx2,
+                                            scattered_router_weights_out=srw2)
+    assert host3 is pageable and torch.equal(pageable, host) and torch.equal(idx2, idx) and torch.equal(sx2, sx)
     saved = sx.clone()
     full_moe.swiglu_expert_loop_fwd(sx, slot.x_up, w_up, w_down, host, primary_stream=stream, secondary_stream=None,
                                     x_act_even=None, x_act_odd=None)

@@ -9,7 +9,8 @@ import torch
 
 from flextrain_amd import ops
 from flextrain_amd.host_memory import (HostMemoryBackend, LocalPinnedHostBackend, destroy_pinned_tensor, pin_tensor)
-from flextrain_amd.optim import AdamW, AdamWHyperparams, flextrain_adamw_step_streamed, state_key
+from flextrain_amd.optim import (AdamW, AdamWHyperparams, adamw_stream_workspace, flextrain_adamw_step_streamed,
+                                 state_key)
 from flextrain_amd.streams import EventBook, StreamBundle
 from oracle import adamw as o_adamw
 from util import gen, randn
@@ -114,6 +115,88 @@ def test_streamed_step_equals_resident_kernel_and_oracle(dev, n, sub, slots, sta
     if state_dtype == torch.float32:
         torch.testing.assert_close(host["m"], m_ref, rtol=1e-4, atol=1e-7)
         torch.testing.assert_close(host["v"], v_ref, rtol=1e-4, atol=1e-10)
+    for t in host.values():
+        be.release(t)
+
+
+def _pinned_state(be, n, seed, step_fill=None):
+    p, gr, m, v = _state(n, seed)
+    host = {}
+    for name, t in (("p", p), ("g", gr), ("m", m), ("v", v)):
+        host[name] = be.allocate_tensor((n,), t.dtype)
+        host[name].copy_(t)
+    host["pc"] = be.allocate_tensor((n,), torch.bfloat16)
+    return (p, gr, m, v), host
+
+
+def _resident(dev, state, step):
+    p, gr, m, v = (t.to(dev) for t in state)
+    pc = torch.empty(p.numel(), dtype=torch.bfloat16, device=dev)
+    ops.flextrain_adamw_step(p, gr, m, v, step=step, params_bf16_out=pc, **HP)
+    return p.cpu(), m.cpu(), v.cpu(), pc.cpu()
+
+
+@pytest.mark.parametrize("raw_workspace", [False, True])
+def test_back_to_back_calls_on_one_workspace_need_no_sync(dev, raw_workspace):
+    """Successive chunks (the engine's layer-after-layer pattern) through ONE staging workspace with
+    nothing between the calls: the second call's copies-in must not overwrite slots the first call's
+    kernels and copies-out still use.  Three chunks of different sizes, each several rounds of the
+    slots, then one more step on the first chunk; every host buffer equals the resident kernel."""
+    be = LocalPinnedHostBackend()
+    sb = StreamBundle.create(dev)
+    sub, slots = 64 * 1024, 3
+    sizes = (1_500_003 // 8 * 8, 700_000, 1_000_003)
+    chunks = [_pinned_state(be, n, 300 + i) for i, n in enumerate(sizes)]
+    ws = adamw_stream_workspace(sub, slots, torch.float32, torch.bfloat16, torch.float32, True, dev)
+    if raw_workspace:
+        ws = ws.buffer                          # no ring: every call fences on compute / outbound instead
+    for state, host in chunks:
+        flextrain_adamw_step_streamed(host["p"], host["g"], host["m"], host["v"], streams=sb, step=4,
+                                      params_bf16_out=host["pc"], workspace=ws, sub_elems=sub, n_slots=slots, **HP)
+    state0, host0 = chunks[0]
+    flextrain_adamw_step_streamed(host0["p"], host0["g"], host0["m"], host0["v"], streams=sb, step=5,
+                                  params_bf16_out=host0["pc"], workspace=ws, sub_elems=sub, n_slots=slots, **HP)
+    sb.synchronize_all()
+    for i, (state, host) in enumerate(chunks):
+        p, m, v, pc = _resident(dev, state, 4)
+        if i == 0:
+            p, m, v, pc = _resident(dev, (p, state[1], m, v), 5)
+        assert torch.equal(host["p"], p) and torch.equal(host["m"], m) and torch.equal(host["v"], v), f"chunk {i}"
+        assert torch.equal(host["pc"], pc), f"chunk {i} bf16 copy"
+    for _, host in chunks:
+        for t in host.values():
+            be.release(t)
+
+
+def test_streamed_step_full_llama_layer_chunk(dev):
+    """218,112,000 parameters (one Llama-3.1-8B decoder layer): fp32 p/m/v + bf16 g in pinned host
+    memory, 3 slots x 4 Mi elements, bf16 copy-out to pinned host.  Bit-equal to the resident kernel
+    on all elements; against the oracle on a strided sample (rtol 1e-4)."""
+    n = 218_112_000
+    be = LocalPinnedHostBackend()
+    g = gen(1003)
+    host = dict(p=be.allocate_tensor((n,), torch.float32), g=be.allocate_tensor((n,), torch.bfloat16),
+                m=be.allocate_tensor((n,), torch.float32), v=be.allocate_tensor((n,), torch.float32),
+                pc=be.allocate_tensor((n,), torch.bfloat16))
+    host["p"].normal_(0, 0.02, generator=g)
+    host["g"].copy_(torch.empty(n).normal_(0, 1e-3, generator=g))
+    host["m"].normal_(0, 1e-3, generator=g)
+    host["v"].normal_(0, 1e-3, generator=g).square_()
+    sample = torch.arange(0, n, 997)
+    before = {k: host[k][sample].clone() for k in ("p", "g", "m", "v")}
+    pd, gd, md, vd = (host[k].to(dev) for k in ("p", "g", "m", "v"))
+    pcd = torch.empty(n, dtype=torch.bfloat16, device=dev)
+    ops.flextrain_adamw_step(pd, gd, md, vd, step=4, params_bf16_out=pcd, **HP)
+    sb = StreamBundle.create(dev)
+    assert flextrain_adamw_step_streamed(host["p"], host["g"], host["m"], host["v"], streams=sb, step=4,
+                                         params_bf16_out=host["pc"], **HP) == 0
+    sb.synchronize_all()
+    for k, d in (("p", pd), ("m", md), ("v", vd), ("pc", pcd)):
+        assert torch.equal(host[k].to(dev), d), k
+    p_ref, m_ref, v_ref, _ = o_adamw.adamw_step(before["p"], before["g"], before["m"], before["v"], step=4, **HP)
+    torch.testing.assert_close(host["p"][sample], p_ref, rtol=1e-4, atol=1e-7)
+    torch.testing.assert_close(host["m"][sample], m_ref, rtol=1e-4, atol=1e-7)
+    torch.testing.assert_close(host["v"][sample], v_ref, rtol=1e-4, atol=1e-10)
     for t in host.values():
         be.release(t)
 

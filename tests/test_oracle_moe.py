@@ -183,3 +183,140 @@ def test_grouped_expert_block_matches_eager_autograd():
     torch.testing.assert_close(dprobs[mapping.reshape(-1).long()].reshape(T, K), gp, rtol=1e-4, atol=1e-5)
     torch.testing.assert_close(g_up, gu, rtol=1e-4, atol=1e-5)
     torch.testing.assert_close(g_down, gd, rtol=1e-4, atol=1e-5)
+
+
+# ------------------------------------------------------------------ whole block
+def _eager_block(x, w_router, w_up, w_down, residual, dy, ids, mode, lb_coef, tokens_per_step, counts, keep=None):
+    """The routed block as one differentiable fp64 expression with the selection held
+    constant (tests/moe/test_moe_backend_parity.py:45-107 for the experts, the router
+    path of flextrain/ops/full_moe.py:306-349 around it): autograd gives every gradient."""
+    T, d = x.shape
+    E, F2, _ = w_up.shape
+    K = ids.shape[1]
+    x = x.double().requires_grad_()
+    w_router = w_router.double().requires_grad_()
+    w_up = w_up.double().requires_grad_()
+    w_down = w_down.double().requires_grad_()
+    logits = x @ w_router
+    ce = ids.long()
+    if mode == "topk_then_softmax":
+        p = torch.softmax(logits.gather(1, ce), -1)
+    else:
+        p = torch.softmax(logits, -1).gather(1, ce)
+    out = residual.double().clone()
+    for t in range(T):
+        for k in range(K):
+            e = int(ce[t, k])
+            if keep is not None and e not in keep:
+                continue
+            pre = w_up[e] @ x[t]
+            h = torch.nn.functional.silu(pre[F2 // 2:]) * pre[:F2 // 2]
+            out = out + torch.nn.functional.one_hot(torch.tensor(t), T).double()[:, None] * (p[t, k] * (w_down[e] @ h))
+    loss = (out * dy.double()).sum()
+    if lb_coef > 0.0 and tokens_per_step is not None:
+        f = counts.double() / (T * K)                                  # a constant of the step
+        loss = loss + lb_coef * E * (f * torch.softmax(logits, -1).sum(0)).sum() / tokens_per_step
+    dx, g_router, g_up, g_down = torch.autograd.grad(loss, (x, w_router, w_up, w_down))
+    return out.detach(), dx, g_router, g_up, g_down
+
+
+def _block_case(seed, T=24, d=16, E=6, F=10, K=3):
+    g = gen(seed)
+    x = randn(g, T, d, dtype=torch.float32)
+    w_router = randn(g, d, E, dtype=torch.float32) * 0.5
+    w_up = randn(g, E, 2 * F, d, dtype=torch.float32) * 0.3
+    w_down = randn(g, E, d, F, dtype=torch.float32) * 0.3
+    residual = randn(g, T, d, dtype=torch.float32)
+    dy = randn(g, T, d, dtype=torch.float32)
+    logits = (x.double() @ w_router.double()).float()
+    return x, w_router, w_up, w_down, residual, dy, logits, K
+
+
+@pytest.mark.parametrize("mode", ["topk_then_softmax", "softmax_then_topk"])
+@pytest.mark.parametrize("lb", [0.0, 0.05])
+def test_routed_block_matches_autograd_of_the_eager_block(mode, lb):
+    x, w_router, w_up, w_down, residual, dy, logits, K = _block_case(11)
+    T = x.shape[0]
+    tps = 2 * T if lb else None
+    got = o_moe.routed_block_fwd_bwd(x, logits, w_router, w_up, w_down, residual, dy, K, mode=mode,
+                                     load_balance_coef=lb, tokens_per_step=tps)
+    out, dx, g_router, g_up, g_down = _eager_block(x, w_router, w_up, w_down, residual, dy, got["ids"], mode, lb,
+                                                   tps, got["counts"])
+    torch.testing.assert_close(got["out"].double(), out, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(got["dx"].double(), dx, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(got["g_router"].double(), g_router, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(got["g_up"].double(), g_up, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(got["g_down"].double(), g_down, rtol=1e-4, atol=1e-5)
+    # the load-balance term must actually move the router path when it is on
+    if lb:
+        off = o_moe.routed_block_fwd_bwd(x, logits, w_router, w_up, w_down, residual, dy, K, mode=mode)
+        assert (off["g_router"] - got["g_router"]).abs().max() > 1e-5
+        torch.testing.assert_close(off["g_up"], got["g_up"], rtol=0, atol=0)
+
+
+def test_routed_block_load_balance_needs_both_arguments():
+    # full_moe.py:327: the aux gradient is added only when the coefficient is positive AND a step size is given
+    x, w_router, w_up, w_down, residual, dy, logits, K = _block_case(12)
+    a = o_moe.routed_block_fwd_bwd(x, logits, w_router, w_up, w_down, residual, dy, K)
+    b = o_moe.routed_block_fwd_bwd(x, logits, w_router, w_up, w_down, residual, dy, K, load_balance_coef=0.05)
+    assert torch.equal(a["dx"], b["dx"]) and torch.equal(a["g_router"], b["g_router"])
+
+
+def test_routed_block_expert_subset_is_the_block_with_the_other_experts_removed():
+    x, w_router, w_up, w_down, residual, dy, logits, K = _block_case(13)
+    keep = (1, 4)
+    full = o_moe.routed_block_fwd_bwd(x, logits, w_router, w_up, w_down, residual, dy, K)
+    sub = o_moe.routed_block_fwd_bwd(x, logits, w_router, w_up, w_down, residual, dy, K, experts=keep)
+    assert torch.equal(sub["ids"], full["ids"]) and torch.equal(sub["mapping"], full["mapping"])
+    assert torch.equal(sub["counts"], full["counts"])
+    assert full["counts"][list(keep)].min() > 0
+    for e in range(w_up.shape[0]):
+        if e in keep:
+            assert torch.equal(sub["g_up"][e], full["g_up"][e]) and torch.equal(sub["g_down"][e], full["g_down"][e])
+            assert sub["g_up"][e].abs().max() > 0
+        else:
+            assert not sub["g_up"][e].any() and not sub["g_down"][e].any()
+    off = o_moe.expert_offsets(full["counts"])
+    for e in range(w_up.shape[0]):
+        rows = slice(int(off[e]), int(off[e + 1]))
+        if e in keep:
+            assert torch.equal(sub["pre"][rows], full["pre"][rows])
+        else:
+            assert not sub["pre"][rows].any()
+    # and as a whole it is the differentiable block with only those experts present
+    out, dx, g_router, g_up, g_down = _eager_block(x, w_router, w_up, w_down, residual, dy, full["ids"],
+                                                   "topk_then_softmax", 0.0, None, full["counts"], keep=keep)
+    torch.testing.assert_close(sub["out"].double(), out, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(sub["dx"].double(), dx, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(sub["g_router"].double(), g_router, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(sub["g_up"].double(), g_up, rtol=1e-4, atol=1e-5)
+
+
+def test_routed_block_rounding_points_in_bf16():
+    # bf16 inputs: out / dx stay within bf16 tolerance of the fp64 block built from the same bf16 values
+    x, w_router, w_up, w_down, residual, dy, _, K = _block_case(14)
+    bf = lambda t: t.to(torch.bfloat16)
+    xb, wrb, wub, wdb, rb, dyb = map(bf, (x, w_router, w_up, w_down, residual, dy))
+    logits = (xb.double() @ wrb.double()).to(torch.bfloat16)
+    got = o_moe.routed_block_fwd_bwd(xb, logits, wrb, wub, wdb, rb, dyb, K)
+    assert got["out"].dtype == torch.bfloat16 and got["dx"].dtype == torch.bfloat16
+    out, dx, g_router, g_up, g_down = _eager_block(xb.float(), wrb.float(), wub.float(), wdb.float(), rb.float(),
+                                                   dyb.float(), got["ids"], "topk_then_softmax", 0.0, None,
+                                                   got["counts"])
+    torch.testing.assert_close(got["out"].double(), out, rtol=2e-2, atol=3e-2)
+    torch.testing.assert_close(got["dx"].double(), dx, rtol=2e-2, atol=3e-2)
+    torch.testing.assert_close(got["g_up"].double(), g_up, rtol=2e-2, atol=3e-2)
+    torch.testing.assert_close(got["g_down"].double(), g_down, rtol=2e-2, atol=3e-2)
+    torch.testing.assert_close(got["g_router"].double(), g_router, rtol=3e-2, atol=5e-2)
+
+
+def test_routed_block_tokens_are_independent():
+    # out[t] and dx[t] depend on token t alone (no load-balance term): the block on a subset of the
+    # tokens gives exactly the rows of the block on all of them.  The full-size GPU test samples tokens this way.
+    x, w_router, w_up, w_down, residual, dy, logits, K = _block_case(15, T=40)
+    full = o_moe.routed_block_fwd_bwd(x, logits, w_router, w_up, w_down, residual, dy, K)
+    tok = torch.tensor([3, 0, 39, 17, 18])
+    sub = o_moe.routed_block_fwd_bwd(x[tok], logits[tok], w_router, w_up, w_down, residual[tok], dy[tok], K)
+    assert torch.equal(sub["ids"], full["ids"][tok])
+    torch.testing.assert_close(sub["out"], full["out"][tok], rtol=1e-6, atol=1e-6)
+    torch.testing.assert_close(sub["dx"], full["dx"][tok], rtol=1e-6, atol=1e-6)
