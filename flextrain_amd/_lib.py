@@ -55,6 +55,9 @@ _SIGNATURES = {
     "fx_moe_sort_ws_bytes": (c_size_t, [c_int64, c_int]),
     "fx_moe_sort": (c_int, [c_void_p, c_int, c_int64, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
                             c_size_t, c_void_p]),
+    "fx_moe_sort_noalloc": (c_int, [c_void_p, c_int, c_int64, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p]),
+    "fx_moe_sort_noalloc_init": (c_int, []),
+    "fx_moe_sort_noalloc_max_words": (c_size_t, []),
     "fx_copy_i32": (c_int, [c_void_p, c_void_p, c_int, c_void_p]),
     "fx_router_gate_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                                    c_int64, c_int, c_int, c_int, c_int, c_int, c_void_p]),

@@ -9,6 +9,8 @@
 // Expert ids, the index mapping and the per-expert counts are integer results
 // and are uniquely determined by those semantics (ties: the smallest expert
 // index wins; the sort is stable in flat (token*K + slot) order).
+#include <mutex>
+
 #include "common.h"
 #include "flexhip.h"
 
@@ -405,6 +407,65 @@ extern "C" int fx_moe_sort(const void* ids, int ids_are_int64, int64_t n_pairs, 
         FX_CHECK_LAUNCH("fx_moe_sort(map)");
     }
     return 0;
+}
+
+// ---- the same sort for callers that may not allocate -----------------------------------------
+// Callers under HIP graph capture, or in loops that must not touch an allocator, cannot lend a
+// workspace sized per call.  This variant keeps the chunk histograms, totals and starts in a
+// fixed array in device memory that is part of the loaded code object (one copy per GPU, held
+// until the process ends).  The array's name is only a host-side handle: kernels get the
+// device address that hipGetSymbolAddress reports for the GPU that is current.
+constexpr size_t SORT_STATIC_WORDS = (size_t)2 * 1024 * 1024 + 1024;          // 8 MiB + 4 KiB
+static __device__ __align__(256) int32_t scratch[SORT_STATIC_WORDS];
+
+namespace {
+constexpr int MAX_DEVICES = 64;
+int32_t* g_scratch_ptr[MAX_DEVICES] = {};
+std::mutex g_scratch_mutex;
+
+// Device address of `scratch` on the current GPU, resolved once per GPU; nullptr on failure.
+int32_t* static_scratch() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+        (void)hipGetLastError();
+        fprintf(stderr, "flexhip: fx_moe_sort_noalloc: cannot tell the current device\n");
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            (void)hipGetLastError();
+            fprintf(stderr, "flexhip: fx_moe_sort_noalloc: hipGetSymbolAddress failed on device %d: %s\n", dev,
+                    hipGetErrorString(e));
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = reinterpret_cast<int32_t*>(p);
+    }
+    return g_scratch_ptr[dev];
+}
+}  // namespace
+
+extern "C" size_t fx_moe_sort_noalloc_max_words(void) { return SORT_STATIC_WORDS; }
+
+extern "C" int fx_moe_sort_noalloc_init(void) { return static_scratch() ? 0 : -1; }
+
+extern "C" int fx_moe_sort_noalloc(const void* ids, int ids_are_int64, int64_t n_pairs, int E, void* index_out,
+                                   int index_is_int64, int32_t* counts_out, int32_t* counts_host,
+                                   hipStream_t stream) {
+    if (n_pairs < 0 || E <= 0) FX_FAIL("fx_moe_sort_noalloc: bad shape n=%lld E=%d", (long long)n_pairs, E);
+    const size_t need = fx_moe_sort_ws_bytes(n_pairs > 0 ? n_pairs : 1, E);
+    if (need > SORT_STATIC_WORDS * sizeof(int32_t))
+        FX_FAIL("fx_moe_sort_noalloc: %lld pairs over %d experts need %zu bytes of scratch, the built-in array holds "
+                "%zu (E * ceil(n / 256) + 2 E <= %zu words); use fx_moe_sort with a workspace",
+                (long long)n_pairs, E, need, SORT_STATIC_WORDS * sizeof(int32_t), SORT_STATIC_WORDS);
+    int32_t* ws = static_scratch();
+    if (!ws) return -1;
+    // every word the kernels read was written earlier in the same call (chunk histograms by the
+    // histogram kernel, totals by the scan, starts by the starts kernel): nothing needs clearing
+    return fx_moe_sort(ids, ids_are_int64, n_pairs, E, index_out, index_is_int64, counts_out, counts_host, ws,
+                       SORT_STATIC_WORDS * sizeof(int32_t), stream);
 }
 
 extern "C" int fx_copy_i32(const int32_t* src_dev, int32_t* dst, int n, hipStream_t stream) {

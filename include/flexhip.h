@@ -148,6 +148,22 @@ int fx_moe_sort(const void* ids, int ids_are_int64, int64_t n_pairs, int E, void
                 int index_is_int64, int32_t* counts_out, int32_t* counts_host, void* ws, size_t ws_bytes,
                 hipStream_t stream);
 
+/* No counterpart in the reference.  fx_moe_sort for callers that cannot allocate device memory or
+ * lend a workspace sized per call: code under HIP graph capture, tight serving loops, harnesses
+ * that forbid allocation.  Same arguments and results as fx_moe_sort without `ws`: the chunk
+ * histograms, totals and starts live in a fixed device array inside the library (8 MiB + 4 KiB per
+ * GPU, held until the process ends).  Limit: E * ceil(n_pairs / 256) + 2 * E <=
+ * fx_moe_sort_noalloc_max_words() (= 2 * 1024 * 1024 + 1024, e.g. 1 Mi pairs over 512 experts);
+ * larger problems return -1 with a message.  Calls no allocator.  All calls on one GPU share that
+ * GPU's array: calls that overlap on one GPU (different streams, or threads) race; calls on one
+ * stream are ordered and need nothing cleared between them.  fx_moe_sort_noalloc_init() resolves
+ * the array's device address for the current GPU ahead of time (it is otherwise resolved on the
+ * first call on each GPU, which must then happen outside graph capture). */
+size_t fx_moe_sort_noalloc_max_words(void);
+int fx_moe_sort_noalloc_init(void);
+int fx_moe_sort_noalloc(const void* ids, int ids_are_int64, int64_t n_pairs, int E, void* index_out,
+                        int index_is_int64, int32_t* counts_out, int32_t* counts_host, hipStream_t stream);
+
 /* flextrain_copy_expert_counts (flextrain/ops/_kernels/moe.py:787-834; kernel
  * :498-505): a kernel copies n int32 from device memory to dst, which may be
  * pinned host memory (zero-copy store). */
