@@ -20,7 +20,10 @@ def _positions(kind, T, g):
 
 
 @pytest.mark.parametrize("kind", ["arange", "packed", "continuation", "random"])
-@pytest.mark.parametrize("T,Hq,Hk,D", [(512, 32, 8, 128), (100, 4, 4, 64), (33, 3, 1, 256), (7, 1, 1, 16)])
+@pytest.mark.parametrize("T,Hq,Hk,D", [(512, 32, 8, 128), (100, 4, 4, 64), (33, 3, 1, 256), (7, 1, 1, 16),
+                                       (37, 6, 6, 128),      # 3 chunks of 64 packs per token: a wave's two chunks straddle tokens
+                                       (101, 4, 4, 64),      # one chunk per token, odd chunk count
+                                       (19, 5, 2, 128)])     # 7 heads: not a whole number of 64-pack chunks (workgroup kernel)
 def test_fwd_bwd_fused(dev, kind, T, Hq, Hk, D):
     g = gen(1010)
     q, k = randn(g, T, Hq, D), randn(g, T, Hk, D)
