@@ -30,38 +30,65 @@ FX_DEV void adam_elem(float& p, float g, float& m, float& v, const AdamScalars& 
     p = p - a.lr * (mh / denom);
 }
 
-template <typename TP, typename TG, typename TS, bool COPY, bool NT, int UNROLL, bool NTS>
+// N consecutive elements of T (N * sizeof(T) = 8 or 16 bytes, address aligned to that) <-> fp32 registers.
+template <typename T, int N, bool NT>
+FX_DEV void load_n(const T* __restrict__ p, float (&out)[N]) {
+    typedef T V __attribute__((ext_vector_type(N)));
+    V v;
+    if (NT) v = __builtin_nontemporal_load(reinterpret_cast<const V*>(p));
+    else v = *reinterpret_cast<const V*>(p);
+#pragma unroll
+    for (int j = 0; j < N; ++j) out[j] = (float)v[j];
+}
+template <typename T, int N, bool NT>
+FX_DEV void store_n(T* __restrict__ p, const float (&in)[N]) {
+    typedef T V __attribute__((ext_vector_type(N)));
+    V v;
+#pragma unroll
+    for (int j = 0; j < N; ++j) v[j] = (T)in[j];
+    if (NT) __builtin_nontemporal_store(v, reinterpret_cast<V*>(p));
+    else *reinterpret_cast<V*>(p) = v;
+}
+
+// A lane owns UNROLL groups of N consecutive elements, N = 4 when any buffer is fp32 (16-byte
+// accesses to the fp32 buffers, 8-byte ones to 2-byte buffers) and 8 when all are 2-byte.  Lanes of
+// a wave touch consecutive groups, so every load or store instruction of a wave covers one
+// contiguous 512- or 1024-byte run (with 8 fp32 elements per lane each instruction would touch
+// every other 16 bytes).
+template <typename TP, typename TG, typename TS, bool COPY, bool NT, int UNROLL, int N>
 __global__ __launch_bounds__(ADAM_THREADS) void adamw_kernel(
     TP* __restrict__ P, const TG* __restrict__ G, TS* __restrict__ M, TS* __restrict__ V,
     bf16* __restrict__ PCOPY, int64_t n, AdamScalars a) {
-    const int64_t base = (int64_t)blockIdx.x * ADAM_THREADS * 8 * UNROLL;
-    float p[UNROLL][8], g[UNROLL][8], m[UNROLL][8], v[UNROLL][8];
+    const int64_t base = (int64_t)blockIdx.x * ADAM_THREADS * N * UNROLL;
+    float p[UNROLL][N], g[UNROLL][N], m[UNROLL][N], v[UNROLL][N];
     bool full[UNROLL];
-    // p, m, v are rewritten in place: plain loads (non-temporal ones halve the rate of such
-    // read-modify-write streams); g is read once and the bf16 copy is written once
+    // NT (launches that move more than the caches keep): every access is non-temporal.  On the
+    // 218 M-parameter chunk that is 5.75-5.8 TB/s against 5.5 TB/s with plain accesses; it only pays
+    // with whole-run accesses (when an instruction touched every other 16 bytes, the other halves
+    // of the lines were fetched from L2 a second time and non-temporal was the slower variant).
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-        const int64_t off = base + ((int64_t)u * ADAM_THREADS + threadIdx.x) * 8;
-        full[u] = off + 8 <= n;
+        const int64_t off = base + ((int64_t)u * ADAM_THREADS + threadIdx.x) * N;
+        full[u] = off + N <= n;
         if (full[u]) {
-            load_f32<TP, 8>(P + off, p[u]);
-            load_f32<TG, 8, NT>(G + off, g[u]);
-            load_f32<TS, 8>(M + off, m[u]);
-            load_f32<TS, 8>(V + off, v[u]);
+            load_n<TP, N, NT>(P + off, p[u]);
+            load_n<TG, N, NT>(G + off, g[u]);
+            load_n<TS, N, NT>(M + off, m[u]);
+            load_n<TS, N, NT>(V + off, v[u]);
         }
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-        const int64_t off = base + ((int64_t)u * ADAM_THREADS + threadIdx.x) * 8;
+        const int64_t off = base + ((int64_t)u * ADAM_THREADS + threadIdx.x) * N;
         if (full[u]) {
 #pragma unroll
-            for (int j = 0; j < 8; ++j) adam_elem(p[u][j], g[u][j], m[u][j], v[u][j], a);
-            store_f32<TP, 8, NTS>(P + off, p[u]);
-            store_f32<TS, 8, NTS>(M + off, m[u]);
-            store_f32<TS, 8, NTS>(V + off, v[u]);
-            if (COPY) store_f32<bf16, 8, NT>(PCOPY + off, p[u]);
+            for (int j = 0; j < N; ++j) adam_elem(p[u][j], g[u][j], m[u][j], v[u][j], a);
+            store_n<TP, N, NT>(P + off, p[u]);
+            store_n<TS, N, NT>(M + off, m[u]);
+            store_n<TS, N, NT>(V + off, v[u]);
+            if (COPY) store_n<bf16, N, NT>(PCOPY + off, p[u]);
         } else {
-            for (int64_t i = off; i < n && i < off + 8; ++i) {
+            for (int64_t i = off; i < n && i < off + N; ++i) {
                 float pp = (float)P[i], gg = (float)G[i], mm = (float)M[i], vv = (float)V[i];
                 adam_elem(pp, gg, mm, vv, a);
                 P[i] = (TP)pp;
@@ -94,12 +121,13 @@ static void launch_adamw(void* p, const void* g, void* m, void* v, void* pcopy, 
     TS* V = reinterpret_cast<TS*>(v);
     bf16* C = reinterpret_cast<bf16*>(pcopy);
     const bool nt = (size_t)n * (2 * sizeof(TP) + sizeof(TG) + 4 * sizeof(TS)) >= kStreamingBytes;
-#define GO(U, NTS_) { const int64_t per = (int64_t)ADAM_THREADS * 8 * U; const unsigned grid = (unsigned)((n + per - 1) / per); \
-    if (pcopy && nt) adamw_kernel<TP, TG, TS, true, true, U, NTS_><<<grid, ADAM_THREADS, 0, s>>>(P, G, M, V, C, n, a); \
-    else if (pcopy) adamw_kernel<TP, TG, TS, true, false, U, NTS_><<<grid, ADAM_THREADS, 0, s>>>(P, G, M, V, C, n, a); \
-    else if (nt) adamw_kernel<TP, TG, TS, false, true, U, NTS_><<<grid, ADAM_THREADS, 0, s>>>(P, G, M, V, C, n, a); \
-    else adamw_kernel<TP, TG, TS, false, false, U, NTS_><<<grid, ADAM_THREADS, 0, s>>>(P, G, M, V, C, n, a); }
-    GO(1, false)
+    constexpr int N = (sizeof(TP) == 4 || sizeof(TG) == 4 || sizeof(TS) == 4) ? 4 : 8;
+#define GO(U) { const int64_t per = (int64_t)ADAM_THREADS * N * U; const unsigned grid = (unsigned)((n + per - 1) / per); \
+    if (pcopy && nt) adamw_kernel<TP, TG, TS, true, true, U, N><<<grid, ADAM_THREADS, 0, s>>>(P, G, M, V, C, n, a); \
+    else if (pcopy) adamw_kernel<TP, TG, TS, true, false, U, N><<<grid, ADAM_THREADS, 0, s>>>(P, G, M, V, C, n, a); \
+    else if (nt) adamw_kernel<TP, TG, TS, false, true, U, N><<<grid, ADAM_THREADS, 0, s>>>(P, G, M, V, C, n, a); \
+    else adamw_kernel<TP, TG, TS, false, false, U, N><<<grid, ADAM_THREADS, 0, s>>>(P, G, M, V, C, n, a); }
+    GO(1)
 #undef GO
 }
 
