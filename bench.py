@@ -168,6 +168,16 @@ def run_rmsnorm(torch, ops, dev, stream, rn):
              for s in sets]
     ms = _time_launches(torch, stream, bwd_e, warmup=NSETS, reps=4 * NSETS)
     rows.append(_op_entry("c1.rmsnorm_bwd(dX+=,dW+=,y)", 5 * T * D * 2 + D * 2 + T * 4 + 2 * D * 4, "GB/s", ms))
+    # yardstick at this size (16.8 MB per tensor): an elementwise kernel with one read and one write stream, and
+    # the same with three reads and one write (the traffic of the backward), through the same rotating sets
+    with torch.cuda.stream(stream):
+        ms = _time_launches(torch, stream, [lambda s=s: torch.mul(s["x"], 2.0, out=s["y"]) for s in sets], warmup=NSETS, reps=4 * NSETS)
+        rows.append(_op_entry("c1.yardstick: y = 2x over one [2048,4096] tensor (torch elementwise kernel, comparison)",
+                              2 * T * D * 2, "GB/s", ms))
+        ms = _time_launches(torch, stream, [lambda s=s: torch.addcmul(s["dx"], s["x"], s["dy"], out=s["dx"]) for s in sets],
+                            warmup=NSETS, reps=4 * NSETS)
+        rows.append(_op_entry("c1.yardstick: dx += x * dy over [2048,4096] tensors (torch elementwise kernel, comparison)",
+                              4 * T * D * 2, "GB/s", ms))
     del sets, fwd, bwd, bwd_e
     torch.cuda.empty_cache()
     # ---- the same kernels at the token count of the headline workload's layer input x 4 (32768 rows, 268 MB per
@@ -354,7 +364,13 @@ def run_lm_head(torch, dev, stream, rn):
     loss = torch.empty(chunk, dtype=torch.float32, device=dev)
     ms = _time_launches(torch, stream, [lambda: ops.flextrain_softmax_cross_entropy(logits, lab, L=loss)], warmup=2, reps=10)
     # two reads and one write of the logits chunk (the row does not stay in registers at V = 128256)
-    rows.append(_op_entry("c3.softmax_ce [1024,128256] in place", 3 * chunk * V * 2, "GB/s", ms))
+    row = _op_entry("c3.softmax_ce [1024,128256] in place", 3 * chunk * V * 2, "GB/s", ms)
+    # the same launch priced by the least any implementation must move (one read, one write of the chunk)
+    minimal = _op_entry("", 2 * chunk * V * 2, "GB/s", ms)
+    row["bytes_counted"] = "two reads + one write of the logits chunk (what this kernel requests)"
+    row["achieved_by_minimal_bytes"] = minimal["achieved"]
+    row["frac_by_minimal_bytes"] = minimal["frac"]
+    rows.append(row)
     del w, g_store, logits, x, x0
     torch.cuda.empty_cache()
     return rows
@@ -594,12 +610,132 @@ def run_moe(torch, dev, stream, rn):
     act = torch.randn(TK, F, device=dev).to(bf)
     ms = _time_launches(torch, stream, [lambda: flextrain_grouped_gemm_rows(sx, weights["w_up"].transpose(1, 2), counts, pre)],
                         warmup=2, reps=10)
-    rows.append(_op_entry("c5.grouped up-proj [65536,2048]x128x[2048,1536]", 2 * TK * d * 2 * F, "TFLOP/s", ms))
+    def floor(row, flop, nbytes):
+        # the least time the launch can take: its MFMA work at the published peak, or its HBM bytes
+        # (operands and results once, accumulated gradients read and written) at 8 TB/s
+        row["floor_ms"] = round(max(flop / (BF16_PEAK_TFLOPS * 1e12), nbytes / (HBM_PEAK_GBPS * 1e9)) * 1e3, 4)
+        row["floor_bound"] = "mfma" if flop / (BF16_PEAK_TFLOPS * 1e12) >= nbytes / (HBM_PEAK_GBPS * 1e9) else "hbm"
+        row["hbm_bytes"] = nbytes
+        return row
+
+    rows.append(floor(_op_entry("c5.grouped up-proj [65536,2048]x128x[2048,1536]", 2 * TK * d * 2 * F, "TFLOP/s", ms),
+                      2 * TK * d * 2 * F, 2 * (TK * d + E * 2 * F * d + TK * 2 * F)))
     ms = _time_launches(torch, stream, [lambda: flextrain_grouped_gemm_rows(act, weights["w_down"].transpose(1, 2), counts, sx)],
                         warmup=2, reps=10)
-    rows.append(_op_entry("c5.grouped down-proj [65536,768]x128x[768,2048]", 2 * TK * d * F, "TFLOP/s", ms))
+    rows.append(floor(_op_entry("c5.grouped down-proj [65536,768]x128x[768,2048]", 2 * TK * d * F, "TFLOP/s", ms),
+                      2 * TK * d * F, 2 * (TK * F + E * F * d + TK * d)))
     ms = _time_launches(torch, stream, [lambda: flextrain_grouped_gemm_wgrad(pre, sx, grads["g_up"], counts)], warmup=2, reps=10)
-    rows.append(_op_entry("c5.grouped wgrad g_up [1536,T_e]x[T_e,2048] x128", 2 * TK * d * 2 * F, "TFLOP/s", ms))
+    rows.append(floor(_op_entry("c5.grouped wgrad g_up [1536,T_e]x[T_e,2048] x128 (+= bf16)", 2 * TK * d * 2 * F, "TFLOP/s", ms),
+                      2 * TK * d * 2 * F, 2 * (TK * 2 * F + TK * d + 2 * E * 2 * F * d)))
+    return rows
+
+
+def _cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def _cpu_time(fn, budget_s, max_runs=50):
+    """Median wall time of fn() over as many runs as fit budget_s (at least one, after one warm-up
+    when a run is short)."""
+    t0 = time.perf_counter()
+    fn()
+    first = time.perf_counter() - t0
+    if first > budget_s / 2:
+        return first, 1
+    times = []
+    t_begin = time.perf_counter()
+    while len(times) < 3 or (time.perf_counter() - t_begin < budget_s and len(times) < max_runs):
+        t1 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t1)
+    times.sort()
+    return times[len(times) // 2], len(times)
+
+
+def run_cpu_baselines(torch, only):
+    """The CPU oracle (the eager PyTorch formulas the reference keeps as its own checks, restated under
+    oracle/) timed on this machine's host cores on a bounded sample of each configuration other than
+    the headline one; work is scaled to the sample."""
+    from oracle import adamw as o_adam
+    from oracle import linear_ce as o_ce
+    from oracle import moe as o_moe
+    from oracle import rmsnorm as o_norm
+
+    want = lambda tag: not only or tag in only
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    model = _cpu_model()
+    bf = torch.bfloat16
+    g = torch.Generator().manual_seed(1000)
+    rows = []
+
+    def row(name, work, unit, sec, runs, sample):
+        r = _op_entry(name, work, unit, sec * 1e3)
+        r.update({"cores": torch.get_num_threads(), "cpu_model": model, "kind": "port",
+                  "sample": f"{sample}; median of {runs} run(s), {sec * 1e3:.1f} ms each"})
+        return r
+
+    if want("c1"):
+        T, D = 2048, 4096
+        x = torch.randn(T, D, generator=g).to(bf)
+        w = (1 + 0.02 * torch.randn(D, generator=g)).to(bf)
+        dy = torch.randn(T, D, generator=g).to(bf)
+
+        def c1():
+            _, rstd = o_norm.rmsnorm_fwd(x, w)
+            o_norm.rmsnorm_bwd(dy, x, w, rstd)
+
+        sec, runs = _cpu_time(c1, 3.0)
+        rows.append(row("c1.cpu_baseline rmsnorm fwd+bwd", (2 + 3) * T * D * 2 + 2 * D * 2 + 2 * T * 4 + D * 4, "GB/s", sec, runs,
+                        "CPU oracle on the whole configuration ([2048,4096])"))
+    if want("c3"):
+        Ts, d, V = 1024, 4096, 128256
+        x = torch.randn(Ts, d, generator=g).to(bf)
+        wh = (torch.randn(d, V, generator=g) * 0.02).to(bf)
+        wn = torch.ones(d)
+        lab = torch.randint(0, V, (Ts,), generator=g)
+        lab[torch.rand(Ts, generator=g) < 0.1] = -100
+        sec, runs = _cpu_time(lambda: o_ce.head_forward_backward(x, wn, wh, lab, chunk=1024, loss_scale=1.0 / Ts), 0.0)
+        rows.append(row("c3.cpu_baseline linear cross-entropy fwd+bwd", 6 * Ts * d * V, "TFLOP/s", sec, runs,
+                        "CPU oracle on one 1024-token chunk of the 8192 tokens (fp32 GEMMs over the whole vocabulary)"))
+        del wh, x
+    if want("c4"):
+        n = 218_112_000 // 16
+        p = torch.randn(n, generator=g) * 0.02
+        gr = (torch.randn(n, generator=g) * 1e-3).to(bf)
+        m, v = torch.zeros(n), torch.zeros(n)
+        step = [0]
+
+        def c4():
+            step[0] += 1
+            o_adam.adamw_step(p, gr, m, v, lr=3e-5, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1, step=step[0])
+
+        sec, runs = _cpu_time(c4, 3.0)
+        rows.append(row("c4.cpu_baseline adamw step + bf16 copy-out", 28 * n, "GB/s", sec, runs,
+                        "CPU oracle on 1/16 of the chunk (13,632,000 parameters)"))
+    if want("c5"):
+        T, d, E, K, F = 512, 2048, 8, 8, 768
+        x = torch.randn(T, d, generator=g).to(bf)
+        dy = torch.randn(T, d, generator=g).to(bf)
+        wr = (torch.randn(d, E, generator=g) * 0.02).to(bf)
+        wu = (torch.randn(E, 2 * F, d, generator=g) * 0.02).to(bf)
+        wd = (torch.randn(E, d, F, generator=g) * 0.02).to(bf)
+
+        def c5():
+            logits = (x.float() @ wr.float()).to(bf)
+            o_moe.routed_block_fwd_bwd(x, logits, wr, wu, wd, x, dy, K)
+
+        sec, runs = _cpu_time(c5, 3.0)
+        rows.append(row("c5.cpu_baseline moe block fwd+bwd", 18 * T * K * d * F + 6 * T * d * E, "TFLOP/s", sec, runs,
+                        "CPU oracle on 1/16 of the block: 512 tokens, 8 experts, top-8 (512 rows per expert as in the "
+                        "full block)"))
     return rows
 
 
@@ -715,6 +851,8 @@ def main():
 
     # -------------------------------------------------------- CPU baseline
     cpu = None
+    if not args.no_cpu and not args.no_extra:
+        op_rows += run_cpu_baselines(torch, [t.strip() for t in args.only.split(",") if t.strip()])
     if not args.no_cpu:
         from oracle import glu as o_glu
         from oracle import rope as o_rope
@@ -745,7 +883,7 @@ def main():
         times.sort()
         med = times[len(times) // 2]
         cpu = {"value": round(step_bytes * (Ts / T) / med / 1e9, 3), "unit": "GB/s",
-               "cores": torch.get_num_threads(), "kind": "port",
+               "cores": torch.get_num_threads(), "kind": "port", "cpu_model": _cpu_model(),
                "sample": f"CPU oracle (PyTorch fp32 formulas) on the first {Ts} of {T} tokens of the same "
                          f"workload, median of {len(times)} runs, {med * 1e3:.1f} ms each"}
 

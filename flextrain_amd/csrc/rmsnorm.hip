@@ -65,13 +65,16 @@ __global__ __launch_bounds__(THREADS) void rmsnorm_fwd_kernel(
     const int64_t row = (int64_t)blockIdx.x * G + g;
     const bool row_ok = row < rows;
 
-    float x[MAXV][8];
+    // the weight packs are requested together with the row: fetched after the reduction they
+    // would add a second exposed memory round trip to a kernel that lasts two or three
+    float x[MAXV][8], w[MAXV][8];
     float ss = 0.f;
 #pragma unroll
     for (int v = 0; v < MAXV; ++v) {
         const int col = (v * LPR + l) * 8;
         if (row_ok && col < ncols) {
             load8<T>(X + row * ncols + col, x[v]);
+            if (W != nullptr) load_w8(W, w_dt, col, w[v]);
         } else {
 #pragma unroll
             for (int j = 0; j < 8; ++j) x[v][j] = 0.f;
@@ -95,10 +98,8 @@ __global__ __launch_bounds__(THREADS) void rmsnorm_fwd_kernel(
         if (row_ok && col < ncols) {
             float y[8];
             if (W != nullptr) {
-                float w[8];
-                load_w8(W, w_dt, col, w);
 #pragma unroll
-                for (int j = 0; j < 8; ++j) y[j] = round_to<T>(x[v][j] * rstd) * w[j];
+                for (int j = 0; j < 8; ++j) y[j] = round_to<T>(x[v][j] * rstd) * w[v][j];
             } else {
 #pragma unroll
                 for (int j = 0; j < 8; ++j) y[j] = x[v][j] * rstd;
@@ -180,22 +181,56 @@ __global__ __launch_bounds__(THREADS) void rmsnorm_bwd_kernel(
         if (has_w && col < ncols) load_w8(W, w_dt, col, w[v]);
     }
 
-    for (int it = 0; it < iters; ++it) {
+    // Raw 16-byte packs of the NEXT iteration's x, dy and (when accumulating) old dx are requested
+    // before the current iteration is reduced, and the old dx together with x and dy rather than
+    // after the row reduction: each of those was an exposed memory round trip in a kernel that
+    // makes one or two iterations at small token counts.
+    typedef typename VecOf<T>::type Pack;
+    constexpr int PN = 8 / VecOf<T>::N;     // 16-byte packs per 8 elements
+    Pack xr[MAXV][PN], dyr[MAXV][PN], oldr[MAXV][PN];
+    auto fetch = [&](int it) {
         const int64_t row = ((int64_t)it * gridDim.x + blockIdx.x) * G + g;
-        const bool row_ok = row < rows;
-        float x[MAXV][8], dy[MAXV][8];
-        const float rstd = row_ok ? RSTD[row] : 0.f;
-        float dot = 0.f;
+        const bool ok = row < rows;
 #pragma unroll
         for (int v = 0; v < MAXV; ++v) {
             const int col = (v * LPR + l) * 8;
-            if (row_ok && col < ncols) {
-                load8<T>(X + row * ncols + col, x[v]);
-                load8<T>(DY + row * ncols + col, dy[v]);
-            } else {
+            if (ok && col < ncols) {
 #pragma unroll
-                for (int j = 0; j < 8; ++j) { x[v][j] = 0.f; dy[v][j] = 0.f; }
+                for (int q = 0; q < PN; ++q) {
+                    xr[v][q] = *reinterpret_cast<const Pack*>(X + row * ncols + col + q * VecOf<T>::N);
+                    dyr[v][q] = *reinterpret_cast<const Pack*>(DY + row * ncols + col + q * VecOf<T>::N);
+                    if (accumulate_dx) oldr[v][q] = *reinterpret_cast<const Pack*>(DX + row * ncols + col + q * VecOf<T>::N);
+                }
             }
+        }
+    };
+    constexpr bool AHEAD = MAXV * PN <= 4;  // wider rows of 4-byte elements would spill: they fetch per iteration
+    if (AHEAD && iters > 0) fetch(0);
+    for (int it = 0; it < iters; ++it) {
+        if (!AHEAD) fetch(it);
+        const int64_t row = ((int64_t)it * gridDim.x + blockIdx.x) * G + g;
+        const bool row_ok = row < rows;
+        float x[MAXV][8], dy[MAXV][8];
+        Pack old[MAXV][PN];                       // stays packed until it is added
+        const float rstd = row_ok ? RSTD[row] : 0.f;
+#pragma unroll
+        for (int v = 0; v < MAXV; ++v) {
+            const int col = (v * LPR + l) * 8;
+            const bool ok = row_ok && col < ncols;
+#pragma unroll
+            for (int q = 0; q < PN; ++q)
+#pragma unroll
+                for (int e = 0; e < VecOf<T>::N; ++e) {
+                    x[v][q * VecOf<T>::N + e] = ok ? (float)xr[v][q][e] : 0.f;
+                    dy[v][q * VecOf<T>::N + e] = ok ? (float)dyr[v][q][e] : 0.f;
+                }
+#pragma unroll
+            for (int q = 0; q < PN; ++q) old[v][q] = oldr[v][q];
+        }
+        if (AHEAD && it + 1 < iters) fetch(it + 1);
+        float dot = 0.f;
+#pragma unroll
+        for (int v = 0; v < MAXV; ++v) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const float xh = x[v][j] * rstd;
@@ -215,10 +250,8 @@ __global__ __launch_bounds__(THREADS) void rmsnorm_bwd_kernel(
 #pragma unroll
                 for (int j = 0; j < 8; ++j) dx[j] = rstd * (dy[v][j] - x[v][j] * k);
                 if (accumulate_dx) {
-                    float old[8];
-                    load8<T>(DX + row * ncols + col, old);
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) dx[j] = old[j] + dx[j];
+                    for (int j = 0; j < 8; ++j) dx[j] = (float)old[v][j / VecOf<T>::N][j % VecOf<T>::N] + dx[j];
                 }
                 store8<T>(DX + row * ncols + col, dx);
                 if (YOUT != nullptr) {
@@ -369,9 +402,8 @@ static inline bool pick_cfg(int ncols, NormCfg& c) {
 // Backward workgroup size per config: wide rows keep many registers per lane,
 // so they get fewer waves per workgroup.
 static inline int bwd_threads(const NormCfg& c) {
-    if (c.lpr < 256) return 1024;
-    if (c.maxv <= 2) return 1024;
-    if (c.maxv == 4) return 512;
+    if (c.maxv == 1) return 1024;
+    if (c.maxv <= 4) return 512;     // two packs per lane and the next iteration's requests need 256 registers
     return 256;
 }
 
@@ -424,8 +456,8 @@ static int launch_bwd(const void* dy, const void* x, const void* w, int w_dt, co
         rmsnorm_bwd_kernel<T, L, V, TH><<<nblocks, TH, lds, s>>>(DY, X, w, w_dt, rstd, DX, acc_dx, Y, partial, rows, ncols, iters); \
         return 0;                                                                                 \
     }
-    FX_BWD_CASE(16, 1, 1024) FX_BWD_CASE(32, 1, 1024) FX_BWD_CASE(64, 1, 1024) FX_BWD_CASE(64, 2, 1024)
-    FX_BWD_CASE(256, 1, 1024) FX_BWD_CASE(256, 2, 1024) FX_BWD_CASE(256, 4, 512) FX_BWD_CASE(256, 8, 256)
+    FX_BWD_CASE(16, 1, 1024) FX_BWD_CASE(32, 1, 1024) FX_BWD_CASE(64, 1, 1024) FX_BWD_CASE(64, 2, 512)
+    FX_BWD_CASE(256, 1, 1024) FX_BWD_CASE(256, 2, 512) FX_BWD_CASE(256, 4, 512) FX_BWD_CASE(256, 8, 256)
 #undef FX_BWD_CASE
     return -1;
 }
