@@ -49,7 +49,7 @@ def _parse():
     ap.add_argument("--no-extra", action="store_true", help="skip the non-headline configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--only", default="", help="comma-separated subset of the non-headline configurations "
-                                               "(c1, c3, c4, c5, ffn, attn, act, probe) to run, e.g. for a profiler pass")
+                                               "(c1, c3, c4, c5, ffn, attn, act, disp, probe) to run, e.g. for a profiler pass")
     return ap.parse_args()
 
 
@@ -138,9 +138,54 @@ def run_extra(torch, ops, dev, stream, rn, only):
         rows += run_attention_proj(torch, dev, stream, rn)
     if want("act"):
         rows += run_activation_slots(torch, dev)
+    if want("disp"):
+        rows += run_dispatch_overhead(torch, dev, stream)
     if want("probe"):
         rows += run_hw_probe(torch, dev)
     return rows
+
+
+def run_dispatch_overhead(torch, dev, stream):
+    """Host time per dispatcher call on a GEMM too small to matter (64^3): the validating ``matmul``
+    (ctypes), the class's ``matmul_fast`` (tensor introspection + the C fast-call entry) and the raw
+    24-argument C entry on pre-extracted values; the library's own time per call (cache look-up and
+    kernel launch, from get_stats) is common to all three."""
+    from flextrain_amd import matmul_dispatcher as md
+
+    A = torch.ones(64, 64, dtype=torch.bfloat16, device=dev)
+    D = torch.empty_like(A)
+    disp = md.CublasLtDispatcher()
+    sp = stream.cuda_stream
+    disp.matmul(sp, A, A, D=D)
+    torch.cuda.synchronize()
+    n = 2000
+
+    def per_call(fn):
+        best = 1e9
+        for _ in range(3):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(n):
+                fn()
+            best = min(best, (time.perf_counter() - t0) / n)
+            torch.cuda.synchronize()
+        return best * 1e6
+
+    raw = [disp._ctx_int, sp, 64, 64, 64, A.data_ptr(), 64, 0, A.data_ptr(), 64, 0, 0, 64, D.data_ptr(), 64,
+           disp.ws_ptr, disp.workspace_size, 2, 2, 2, 2, 0, 1.0, 0.0]
+    fast = md._bind_fast()
+    st0 = disp.get_stats()
+    us_raw = per_call(lambda: fast(*raw))
+    st1 = disp.get_stats()
+    cpp_us = ((st1["avg_cpp_total_us"] * st1["matmuls_called"] - st0["avg_cpp_total_us"] * st0["matmuls_called"])
+              / max(1, st1["matmuls_called"] - st0["matmuls_called"]))
+    us_fast = per_call(lambda: disp.matmul_fast(sp, A, A, D=D))
+    us_full = per_call(lambda: disp.matmul(sp, A, A, D=D))
+    return [{"op": "disp.host time per dispatcher call (64^3 GEMM, 2000 calls back to back)", "algorithmic": None,
+             "unit": "us", "frac": None, "ms": None, "achieved": None,
+             "matmul_ctypes_us": round(us_full, 2), "matmul_fast_method_us": round(us_fast, 2),
+             "raw_fast_call_entry_us": round(us_raw, 2), "library_time_per_call_us": round(cpp_us, 2),
+             "raw_entry_overhead_over_library_us": round(us_raw - cpp_us, 2)}]
 
 
 def run_rmsnorm(torch, ops, dev, stream, rn):

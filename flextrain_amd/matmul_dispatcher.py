@@ -50,16 +50,29 @@ def dtype_enum(dtype):
         raise ValueError(f"unsupported dtype {dtype} for matmul_fast") from None
 
 
-def matmul_fast(ctx_int, stream, M, N, K, ptr_A, lda, trans_a, ptr_B, ldb, trans_b, ptr_C, ldc, ptr_D, ldd,
-                ws_ptr, ws_bytes, a_dt, b_dt, c_dt, d_dt, compute_dt, alpha, beta):
-    """Raw 24-argument entry with the argument order of the reference's
-    ``matmul_fast`` (helpers/matmul_dispatcher/src/dispatch_pyext.cpp:37-140).
-    Raises ``RuntimeError`` when ``dispatch_matmul`` reports failure."""
-    rc = lib().dispatch_matmul(ctx_int, stream, M, N, K, ptr_A, lda, ptr_B, ldb, ptr_C, ldc, ptr_D, ldd,
-                               ws_ptr, ws_bytes, a_dt, b_dt, c_dt, d_dt, compute_dt, alpha, beta,
-                               trans_a, trans_b)
-    if rc != 0:
-        raise RuntimeError(f"dispatch_matmul failed (rc={rc})")
+_fast_entry = None
+
+
+def _bind_fast():
+    """The C fast-call entry (``flextrain_amd/csrc/pyext/dispatch_fast.c``), bound to the
+    ``dispatch_matmul`` of the library this process has loaded.  Raises when the extension has
+    not been built: there is no slower stand-in behind it."""
+    global _fast_entry
+    if _fast_entry is None:
+        from . import _dispatch_fast      # ImportError when the extension is missing
+        _dispatch_fast.bind(ctypes.cast(lib().dispatch_matmul, ctypes.c_void_p).value)
+        _fast_entry = _dispatch_fast.matmul_fast
+    return _fast_entry
+
+
+def matmul_fast(*args):
+    """Raw 24-argument entry with the argument order and error behaviour of the reference's
+    ``matmul_fast`` (helpers/matmul_dispatcher/src/dispatch_pyext.cpp:37-140): ``TypeError`` for any
+    other argument count, ``RuntimeError`` when ``dispatch_matmul`` reports failure.  After the first
+    call the module attribute IS the C function (no Python frame in between)."""
+    global matmul_fast
+    matmul_fast = _bind_fast()
+    return matmul_fast(*args)
 
 
 class CublasLtDispatcher:
@@ -78,6 +91,7 @@ class CublasLtDispatcher:
         self.bf16 = torch.bfloat16
         self.total_python_ns = 0
         self._ctx_int = int(self.ctx) if self.ctx is not None else 0
+        self._fast = _bind_fast()
 
     def __del__(self):
         if getattr(self, "ctx", None):
@@ -299,6 +313,6 @@ class CublasLtDispatcher:
         d_dt = _dtype_to_enum[D.dtype]
         if self.workspace is None:
             self._ensure_workspace(A.device)
-        matmul_fast(self._ctx_int, stream_ptr, M, N, K, ptr_A, ld_A, trans_a, ptr_B, ld_B, trans_b, ptr_C, ld_C,
-                    ptr_D, ld_D, self.ws_ptr, self.workspace_size, dt, dt, d_dt, d_dt, 0, alpha, beta)
+        self._fast(self._ctx_int, stream_ptr, M, N, K, ptr_A, ld_A, trans_a, ptr_B, ld_B, trans_b, ptr_C, ld_C,
+                   ptr_D, ld_D, self.ws_ptr, self.workspace_size, dt, dt, d_dt, d_dt, 0, alpha, beta)
         return D

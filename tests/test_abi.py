@@ -37,3 +37,30 @@ def test_python_binding_covers_the_header():
 
 def test_version_string():
     assert _lib.lib().fx_version().decode().startswith("flexhip")
+
+
+def test_fast_call_extension_loads_and_keeps_the_reference_conventions():
+    """flextrain_amd._dispatch_fast (the METH_FASTCALL entry of
+    helpers/matmul_dispatcher/src/dispatch_pyext.cpp:37-140): 24 positional arguments or TypeError,
+    ValueError for a null context; bound to the dispatch_matmul of the loaded library."""
+    import pytest
+
+    from flextrain_amd import matmul_dispatcher as md
+
+    fast = md._bind_fast()
+    assert type(fast).__name__ == "builtin_function_or_method"
+    with pytest.raises(TypeError):
+        fast(1, 2, 3)
+    with pytest.raises(TypeError):
+        fast(*([0] * 25))
+    null_ctx = [0, 0, 1, 1, 1, 0, 1, 0, 0, 1, 0, 0, 1, 0, 1, 0, 0, 2, 2, 2, 2, 0, 1.0, 0.0]
+    with pytest.raises(ValueError):
+        fast(*null_ctx)
+    bad = list(null_ctx)
+    bad[2] = "not a number"
+    with pytest.raises(TypeError):
+        fast(*bad)
+    # the module-level name of the reference's raw entry resolves to the same C function
+    with pytest.raises(TypeError):
+        md.matmul_fast(1)
+    assert md.matmul_fast is fast

@@ -357,3 +357,33 @@ def test_sum_of_products_fp16(dev):
     assert disp._ksum_ok(Ad, Bd, None, D)
     disp.matmul_sum(torch.cuda.current_stream().cuda_stream, Ad, Bd, D=D)
     _check(D, _ref_sum(As, Bs), torch.float16)
+
+
+def test_raw_fast_call_entry(dev):
+    """The 24-argument C entry (helpers/matmul_dispatcher/src/dispatch_pyext.cpp:37-140): same bits as
+    matmul, RuntimeError when dispatch_matmul reports failure."""
+    from flextrain_amd import matmul_dispatcher as md
+
+    g = gen(77)
+    A, B = randn(g, 300, 512, std=0.5).to(dev), randn(g, 512, 640, std=0.5).to(dev)
+    disp = CublasLtDispatcher()
+    s = torch.cuda.current_stream().cuda_stream
+    want = disp.matmul(s, A, B)
+    D = torch.zeros_like(want)
+    disp._ensure_workspace(A.device)
+    args = [disp._ctx_int, s, 300, 640, 512, A.data_ptr(), 512, 0, B.data_ptr(), 640, 0, 0, 640, D.data_ptr(), 640,
+            disp.ws_ptr, disp.workspace_size, 2, 2, 2, 2, 0, 1.0, 0.0]
+    assert md.matmul_fast(*args) is None
+    assert torch.equal(D, want)
+    # integer alpha / beta are accepted like floats
+    args[22], args[23] = 1, 0
+    md.matmul_fast(*args)
+    assert torch.equal(D, want)
+    bad = list(args)
+    bad[5] = 0                      # null A: dispatch_matmul returns non-zero
+    with pytest.raises(RuntimeError):
+        md.matmul_fast(*bad)
+    bad = list(args)
+    bad[17] = 1                     # A and B dtypes differ
+    with pytest.raises(RuntimeError):
+        md.matmul_fast(*bad)
