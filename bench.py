@@ -339,12 +339,31 @@ def run_streamed_adamw(torch, dev):
         dst.copy_(src, non_blocking=True)
         torch.cuda.synchronize()
         alone[name] = (time.perf_counter() - t0) * 1e3
+    # what the link gives when both directions carry one plain copy of the same bytes at once: the ceiling of
+    # any overlapped schedule (a direction alone is faster than either direction of a concurrent pair)
+    dbuf2 = torch.empty(h2d, dtype=torch.uint8, device=dev)
+    hbuf2 = be.allocate_tensor((h2d,), torch.uint8)
+    both = []
+    for _ in range(3):
+        sb.synchronize_all()
+        t0 = time.perf_counter()
+        with torch.cuda.stream(sb.inbound):
+            dbuf.copy_(hbuf, non_blocking=True)
+        with torch.cuda.stream(sb.outbound):
+            hbuf2.copy_(dbuf2, non_blocking=True)
+        sb.synchronize_all()
+        both.append((time.perf_counter() - t0) * 1e3)
+    both_ms = sorted(both)[1]
+    be.release(hbuf2)
+    del dbuf2
     row = {"op": "c4.adamw streamed from pinned host (fp32 p/m/v, bf16 g, bf16 copy-out; 3 slots x 4Mi elements)",
            "algorithmic": h2d + d2h, "ms": round(ms, 3), "achieved": round((h2d + d2h) / (ms * 1e-3) / 1e9, 2),
            "unit": "GB/s (host link, both directions summed)", "frac": None,
            "h2d_GBps": round(h2d / (ms * 1e-3) / 1e9, 2), "d2h_GBps": round(d2h / (ms * 1e-3) / 1e9, 2),
            "copy_alone_ms": {k: round(v, 3) for k, v in alone.items()},
-           "overlap_efficiency": round(max(alone.values()) / ms, 4)}
+           "overlap_efficiency": round(max(alone.values()) / ms, 4),
+           "plain_copies_both_directions_at_once_ms": round(both_ms, 3),
+           "frac_of_concurrent_link_ceiling": round(both_ms / ms, 4)}
     for t in host.values():
         be.release(t)
     be.release(hbuf)
@@ -633,11 +652,13 @@ def run_moe(torch, dev, stream, rn):
         full_moe.routed_swiglu_moe_fwd(x, weights, out_tensor=out, residual=x, top_k=K, num_experts=E,
                                        routing_mode="topk_then_softmax", **common)
 
-    def bwd():
+    second = torch.cuda.Stream(device=dev)
+
+    def bwd(secondary=second):
         release()
         full_moe.routed_swiglu_moe_bwd(dy, weights, grads, slot, extra, 0, ffn_norm_output=x, top_k=K, num_experts=E,
                                        routing_mode="topk_then_softmax", load_balance_coef=0.0,
-                                       total_tokens_per_step=None, primary_stream=stream, secondary_stream=None,
+                                       total_tokens_per_step=None, primary_stream=stream, secondary_stream=secondary,
                                        scratch_fn=scratch, expert_compute=backend)
 
     rows = []
@@ -646,7 +667,9 @@ def run_moe(torch, dev, stream, rn):
     ms_f = _time_launches(torch, stream, [fwd], warmup=2, reps=5)
     rows.append(_op_entry("c5.moe block fwd (route+sort+scatter+experts+gather)", fl_fwd, "TFLOP/s", ms_f))
     ms_b = _time_launches(torch, stream, [bwd], warmup=2, reps=5)
-    rows.append(_op_entry("c5.moe block bwd", fl_bwd, "TFLOP/s", ms_b))
+    rows.append(_op_entry("c5.moe block bwd (weight gradients on the secondary stream)", fl_bwd, "TFLOP/s", ms_b))
+    ms_b1 = _time_launches(torch, stream, [lambda: bwd(None)], warmup=2, reps=5)
+    rows.append(_op_entry("c5.moe block bwd, one stream", fl_bwd, "TFLOP/s", ms_b1))
     rows.append(_op_entry("c5.moe block fwd+bwd", fl_fwd + fl_bwd, "TFLOP/s", ms_f + ms_b))
     # the grouped GEMMs alone, on the routing the block just produced
     counts = slot.expert_counts

@@ -127,17 +127,37 @@ def swiglu_expert_loop_bwd(scattered_upstream, scattered_x, x_preact_buf, srw, d
     accumulator missing from ``grads`` (or None) is skipped."""
     TK = scattered_upstream.shape[0]
     counts = _device_counts(expert_counts_cpu, expert_counts_gpu)
+    two = secondary_stream is not None and secondary_stream != primary_stream
     with torch.cuda.stream(primary_stream):
         dx_act = torch.empty((TK, expert_dim), dtype=scattered_upstream.dtype, device=scattered_upstream.device)
         fwd_act = torch.empty_like(dx_act)
         flextrain_grouped_gemm_rows(scattered_upstream, w_down, counts, dx_act)                        # (a)
         flextrain_swiglu_moe_bwd(dx_act, x_preact_buf[:TK], srw[:TK], dx=dx_up_up_grouped[:TK], dw=dprobs[:TK],
                                  fwd_act=fwd_act)                                                       # (b)
+        if two:
+            ready = torch.cuda.Event()
+            ready.record(primary_stream)
+    # The two weight-gradient launches only read what (b) left behind and write the accumulators, so
+    # with a second stream they run beside the dgrad through w_up (the reference alternates its two
+    # streams between experts for the same reason, full_moe.py:420-466); the primary stream waits
+    # for them before this function returns, so every buffer is free for the caller as before.
+    wgrad_stream = secondary_stream if two else primary_stream
+    with torch.cuda.stream(wgrad_stream):
+        if two:
+            wgrad_stream.wait_event(ready)
         if grads.get("g_down") is not None:
             flextrain_grouped_gemm_wgrad(scattered_upstream, fwd_act, grads["g_down"], counts)          # (c)
-        flextrain_grouped_gemm_rows(dx_up_up_grouped[:TK], w_up, counts, dx_pre_grouped[:TK])           # (d)
+        if not two:
+            flextrain_grouped_gemm_rows(dx_up_up_grouped[:TK], w_up, counts, dx_pre_grouped[:TK])       # (d)
         if grads.get("g_up") is not None:
             flextrain_grouped_gemm_wgrad(dx_up_up_grouped[:TK], scattered_x, grads["g_up"], counts)     # (e)
+        if two:
+            done = torch.cuda.Event()
+            done.record(wgrad_stream)
+    if two:
+        with torch.cuda.stream(primary_stream):
+            flextrain_grouped_gemm_rows(dx_up_up_grouped[:TK], w_up, counts, dx_pre_grouped[:TK])       # (d)
+            primary_stream.wait_event(done)
 
 
 def swiglu_expert_loop_recompute_x_up(scattered_x, x_preact_buf, w_up, expert_counts_cpu, *, primary_stream,
