@@ -652,9 +652,7 @@ def run_moe(torch, dev, stream, rn):
         full_moe.routed_swiglu_moe_fwd(x, weights, out_tensor=out, residual=x, top_k=K, num_experts=E,
                                        routing_mode="topk_then_softmax", **common)
 
-    second = torch.cuda.Stream(device=dev)
-
-    def bwd(secondary=second):
+    def bwd(secondary=None):
         release()
         full_moe.routed_swiglu_moe_bwd(dy, weights, grads, slot, extra, 0, ffn_norm_output=x, top_k=K, num_experts=E,
                                        routing_mode="topk_then_softmax", load_balance_coef=0.0,
@@ -667,9 +665,7 @@ def run_moe(torch, dev, stream, rn):
     ms_f = _time_launches(torch, stream, [fwd], warmup=2, reps=5)
     rows.append(_op_entry("c5.moe block fwd (route+sort+scatter+experts+gather)", fl_fwd, "TFLOP/s", ms_f))
     ms_b = _time_launches(torch, stream, [bwd], warmup=2, reps=5)
-    rows.append(_op_entry("c5.moe block bwd (weight gradients on the secondary stream)", fl_bwd, "TFLOP/s", ms_b))
-    ms_b1 = _time_launches(torch, stream, [lambda: bwd(None)], warmup=2, reps=5)
-    rows.append(_op_entry("c5.moe block bwd, one stream", fl_bwd, "TFLOP/s", ms_b1))
+    rows.append(_op_entry("c5.moe block bwd", fl_bwd, "TFLOP/s", ms_b))
     rows.append(_op_entry("c5.moe block fwd+bwd", fl_fwd + fl_bwd, "TFLOP/s", ms_f + ms_b))
     # the grouped GEMMs alone, on the routing the block just produced
     counts = slot.expert_counts

@@ -66,6 +66,7 @@ _SIGNATURES = {
     "fx_moe_scatter": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int64, c_int, c_int,
                                c_int64, c_int, c_void_p]),
     "fx_moe_scatter_weights": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int, c_void_p]),
+    "fx_moe_row_sources": (c_int, [c_void_p, c_int, c_int64, c_int, c_void_p, c_void_p]),
     "fx_moe_gather": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
                               c_int64, c_int, c_int, c_int, c_void_p]),
     "fx_swiglu_moe_fwd": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int64, c_int, c_int64,
@@ -85,7 +86,7 @@ _SIGNATURES = {
                                       c_size_t, c_void_p]),
     "fx_grouped_gemm_rows_glu": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int, c_int64, c_void_p,
                                          c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int, c_int64, c_int,
-                                         c_int, c_int, c_int, c_void_p, c_size_t, c_void_p]),
+                                         c_int, c_int, c_int, c_void_p, c_size_t, c_void_p, c_int64, c_void_p]),
     "fx_gemm_dual_glu": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int, c_void_p, c_void_p, c_int64,
                                  c_void_p, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "fx_gemm_segments": (c_int, [c_void_p, c_int64, c_int, c_int, POINTER(c_void_p), POINTER(c_int64), c_int,

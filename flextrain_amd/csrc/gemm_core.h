@@ -45,6 +45,9 @@ struct OperandView {
     // indices origin + [half, 2 half) of `base` again, and so on.
     int half = 0;
     const T* base2 = nullptr;
+    // Gathered rows (K-contiguous A tiles of the loaders that say so): tile row r is row
+    // row_map[origin + r] of `base` instead of row origin + r.
+    const int32_t* row_map = nullptr;
     // tile row -> which matrix, and the index offset from `origin`
     __device__ __forceinline__ bool dual_second(int r) const { return (r & half) != 0; }
     __device__ __forceinline__ int dual_index(int r) const { return ((r & ~(2 * half - 1)) >> 1) + (r & (half - 1)); }

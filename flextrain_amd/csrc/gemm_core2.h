@@ -278,7 +278,13 @@ struct MmaPipe {
 // address), s_mov m0, s_nop, global_load_lds.  With per-lane 64-bit pointers every load carried
 // about ten vector instructions between the MFMAs (measured: +3 % with two waves per SIMD, +6-8 %
 // with one).  Needs `wave` to be uniform (readfirstlane) and 256 * ld * sizeof(T) < 4 GB.
-FX_DEV void load_to_lds16_s(unsigned lane_off, const void* sbase, unsigned lds_addr) {
+FX_DEV void load_to_lds16_s(unsigned lane_off, const void* sbase_in, unsigned lds_addr) {
+    // the base is wave-uniform by construction; saying so keeps it in scalar registers where the
+    // compiler cannot prove it (a no-op where it can)
+    const uint64_t u = reinterpret_cast<uint64_t>(sbase_in);
+    const void* sbase = reinterpret_cast<const void*>(
+        ((uint64_t)(unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(u >> 32)) << 32) |
+        (uint64_t)(unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)u));   // the builtin returns a signed int: widen as unsigned
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(lane_off), "s"(sbase) : "memory", "m0");
 }
 
@@ -297,14 +303,18 @@ struct TileLoader {
         half = op.half;
         if (!MN) {
             const int rr = lane >> 3, pos = lane & 7;
+            const bool gathered = !DUAL && op.row_map != nullptr;      // wave-uniform
 #pragma unroll
             for (int j = 0; j < NI; ++j) {
                 const int r = (j * NW + wave) * 8 + rr;
                 int g = op.origin + (DUAL ? op.dual_index(r) : r);
                 g = g < op.ext ? g : op.ext - 1;
-                off[j] = (unsigned)(((int64_t)(g - op.origin) * op.ld + (pos ^ swz(r)) * 8) * (int64_t)sizeof(T));
+                // gathered: the offset is taken from the start of the source matrix (the caller checks
+                // that the whole source stays below 4 GB)
+                const int64_t row = gathered ? (int64_t)op.row_map[g] : (int64_t)(g - op.origin);
+                off[j] = (unsigned)((row * op.ld + (pos ^ swz(r)) * 8) * (int64_t)sizeof(T));
             }
-            base = op.base + (int64_t)op.origin * op.ld;
+            base = gathered ? op.base : op.base + (int64_t)op.origin * op.ld;
             base2 = DUAL ? op.base2 + (int64_t)op.origin * op.ld : nullptr;
             step = GEMM_BK;
         } else {
@@ -380,7 +390,11 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 template <int NW, int WN>
 constexpr size_t epilogue_lds_bytes() { return (size_t)NW * 32 * (WN + 4) * sizeof(float); }
 
-template <typename T, typename TD, int WM, int WN>
+// LOADS_LAND: the caller has requested the first K-step of its next tile before this epilogue; all
+// loads issued so far are waited for just before the last band's stores go out (a wait placed after
+// the epilogue would also wait for every store to drain, because loads and stores share one counter:
+// here the earlier bands' stores have had most of the epilogue to complete).
+template <typename T, typename TD, int WM, int WN, bool LOADS_LAND = false>
 FX_DEV void epilogue_tile(f32x16_t (&acc)[WM / 32][WN / 32], const TD* C, TD* D, int64_t ldc, int64_t ldd, int row_base,
                           int col_base, int M, int N, float alpha, float beta, T* smem, int wave, int lane) {
     constexpr int TM = WM / 32, TN = WN / 32;
@@ -423,6 +437,7 @@ FX_DEV void epilogue_tile(f32x16_t (&acc)[WM / 32][WN / 32], const TD* C, TD* D,
                 const f32x4_t q = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
                 *reinterpret_cast<f32x4_t*>(stage + (lane & 31) * PITCH + j * 32 + 8 * g + 4 * (lane >> 5)) = q;
             }
+        if (LOADS_LAND && i == TM - 1) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         // a wave reads back only what it wrote itself; its LDS accesses complete in order
 #pragma unroll
         for (int t = 0; t < PER_LANE; ++t) {
@@ -470,115 +485,142 @@ constexpr size_t gemm2_lds_bytes() {
 // second matrix (OperandView::half); K must then be a multiple of 64.
 // ZERO = false: `acc` already holds partial sums and is added to (a product summed over several
 // operand pairs, one call per pair; the call ends with a barrier, so the next may start at once).
+//
+// The loop is an object with two halves so that a workgroup that walks several tiles can request
+// the first K-step of its NEXT tile before it runs the epilogue of the current one:
+//   begin(A, B, K, buf0)            set up the loaders, issue the loads of K-step 0 into buf0
+//   finish(A, B, K, buf0, buf1, acc) issue K-step 1 into buf1, run the K loop, end with a barrier
+// Between the two the caller may do anything that leaves buf0 alone and issues no inline-assembly
+// loads of its own (compiler-generated loads and stores are fine: the counted waits below only
+// assume that loads complete in the order they were issued).
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_MN, bool B_MN, bool B_DUAL = false, bool ZERO = true>
+struct MainLoop2 {
+    static constexpr int NW = WAVES_M * WAVES_N, NT = NW * 64;
+    static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+    static constexpr int TM = WM / 32, TN = WN / 32;
+    static constexpr int BUF = (BM + BN) * GEMM_BK;
+    typedef MmaPipe<T, BM, BN, WM, WN, A_MN, B_MN> Pipe;
+    typedef TileLoader<T, BM, NW, A_MN, false> LoadA;
+    typedef typename std::conditional<(B_MN && B_DUAL), TileLoaderV<T, BN, NW, B_MN, B_DUAL>,
+                                      TileLoader<T, BN, NW, B_MN, B_DUAL>>::type LoadB;
+    static constexpr int LD = LoadA::NI + LoadB::NI;            // load instructions per wave and K-step
+    static constexpr int PER = (LD + Pipe::MFMAS - 1) / Pipe::MFMAS;
+    static_assert(GEMM_BK == 64, "the pipeline below is written out for four sub-steps per K-step");
+    static_assert((size_t)2 * BUF * sizeof(T) <= 160 * 1024, "tile configuration exceeds the 160 KB of LDS");
+    LoadA la;
+    LoadB lb;
+    int wave;
+
+    // instruction IDX of the next K-step into the stage at `buf` (K-steps are issued in order)
+    template <int IDX>
+    FX_DEV void issue_one(T* buf) {
+        if constexpr (IDX < LoadA::NI) la.template issue<IDX>(buf, wave);
+        else if constexpr (IDX < LD) lb.template issue<IDX - LoadA::NI>(buf + BM * GEMM_BK, wave);
+    }
+    FX_DEV void issue(T* buf) { static_for<0, LD>([&](auto idx) { issue_one<decltype(idx)::value>(buf); }); }
+
+    FX_DEV void begin(const OperandView<T>& A, const OperandView<T>& B, int K, T* buf0) {
+        const int lane = threadIdx.x & 63;
+        wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // uniform: LDS addresses of the loads stay scalar
+        if (K >= GEMM_BK) {
+            la.init(A, wave, lane);
+            lb.init(B, wave, lane);
+            issue(buf0);
+        }
+    }
+
+    // first_landed: the caller has already waited for the loads of K-step 0 and passed a barrier since
+    FX_DEV void finish(const OperandView<T>& A, const OperandView<T>& B, int K, T* buf0, T* buf1, f32x16_t (&acc)[TM][TN],
+                       bool first_landed = false) {
+        const int tid = threadIdx.x;
+        const int lane = tid & 63;
+        const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+        if (ZERO) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+        }
+        const int nfull = K / GEMM_BK;  // K-steps that need no zero fill
+        // wave-uniform: does any element of this wave's sub-tile lie inside the matrices?
+        const bool live = __builtin_amdgcn_readfirstlane(
+            (A.origin + wm * WM < A.ext) && (B_DUAL || B.origin + wn * WN < B.ext));
+        auto stage = [&](int kt) { return (kt & 1) ? buf1 : buf0; };
+        if (nfull > 0) {
+            typename Pipe::Slot f0, f1;
+            const int ra = wm * WM, rb = wn * WN;
+            // both buffers are free at the start of a tile: the first two K-steps are in flight together
+            // and only the first is waited for (short-K tiles spend a visible share of their time here)
+            if (nfull > 1) issue(buf1);
+            if (!first_landed) {
+                if (nfull > 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LD) : "memory");
+                else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();
+            }
+            if (!live) {
+                // no row (or column) of this wave's sub-tile exists: it keeps loading its share of the
+                // stages and meets every barrier of the loop below, and leaves the matrix cores of its
+                // SIMD to the wave it shares them with (the last row tile of an expert is mostly this)
+                for (int kt = 0; kt + 1 < nfull; ++kt) {
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                    __syncthreads();
+                    if (kt + 2 < nfull) issue(stage(kt));
+                }
+            } else {
+            Pipe::fetch_all(f0, buf0, buf0 + BM * GEMM_BK, 0, ra, rb, lane);
+            for (int kt = 0; kt + 1 < nfull; ++kt) {
+                T* cur = stage(kt);
+                T* nxt = stage(kt + 1);
+                T* curb = cur + BM * GEMM_BK;
+                Pipe::template sub<true>(acc, f0, f1, cur, curb, 1, ra, rb, lane);
+                Pipe::template sub<true>(acc, f1, f0, cur, curb, 2, ra, rb, lane);
+                Pipe::template sub<true>(acc, f0, f1, cur, curb, 3, ra, rb, lane);
+                // Every read of `cur` has been issued.  Once they and this wave's loads of step kt+1 have
+                // landed, the barrier makes `nxt` readable and `cur` writable for everyone; the MFMAs of
+                // the last sub-step then run while the first fragments of step kt+1 are read and the
+                // loads of step kt+2 are issued into `cur`, PER of them after each MFMA (measured 2-3 %
+                // faster in every layout than issuing them in one burst after the barrier).
+                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                __syncthreads();
+                const bool more = kt + 2 < nfull;
+                Pipe::template sub<true>(acc, f1, f0, nxt, nxt + BM * GEMM_BK, 0, ra, rb, lane, [&](auto m) {
+                    constexpr int M = decltype(m)::value;
+                    if (more) static_for<M * PER, (M + 1) * PER>([&](auto idx) { issue_one<decltype(idx)::value>(cur); });
+                });
+            }
+            {   // last full K-step: nothing follows it in these buffers
+                T* cur = stage(nfull - 1);
+                T* curb = cur + BM * GEMM_BK;
+                Pipe::template sub<true>(acc, f0, f1, cur, curb, 1, ra, rb, lane);
+                Pipe::template sub<true>(acc, f1, f0, cur, curb, 2, ra, rb, lane);
+                Pipe::template sub<true>(acc, f0, f1, cur, curb, 3, ra, rb, lane);
+                Pipe::template sub<false>(acc, f1, f0, cur, curb, 0, ra, rb, lane);
+            }
+            }
+        }
+        if (!B_DUAL && nfull * GEMM_BK < K) {  // K tail: through registers into the K-contiguous layout, zero-filled past K
+            Staged2<BM, NT> sa;
+            Staged2<BN, NT> sb;
+            T* buf = stage(nfull);
+            stage2_load<T, BM, NT, A_MN>(sa, A, nfull * GEMM_BK, K, tid);
+            stage2_load<T, BN, NT, B_MN>(sb, B, nfull * GEMM_BK, K, tid);
+            stage2_store<T, BM, NT, A_MN>(sa, buf, tid);     // `buf` was last read two steps ago
+            stage2_store<T, BN, NT, B_MN>(sb, buf + BM * GEMM_BK, tid);
+            __syncthreads();
+            if (live) mma_step<T, BM, BN, WM, WN, false, false>(buf, buf + BM * GEMM_BK, wm * WM, wn * WN, lane, acc);
+        }
+        __syncthreads();  // every wave is past its last LDS read: the buffers are free
+    }
+};
+
 template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_MN, bool B_MN, bool B_DUAL = false, bool ZERO = true>
 FX_DEV void gemm_mainloop2(const OperandView<T>& A, const OperandView<T>& B, int K, T* smem,
                            f32x16_t (&acc)[BM / WAVES_M / 32][BN / WAVES_N / 32]) {
-    constexpr int NW = WAVES_M * WAVES_N, NT = NW * 64;
-    constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
-    constexpr int TM = WM / 32, TN = WN / 32;
-    constexpr int BUF = (BM + BN) * GEMM_BK;
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: LDS addresses of the loads stay scalar
-    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
-
-    if (ZERO) {
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-    }
-
-    const int nfull = K / GEMM_BK;  // K-steps that need no zero fill
-    static_assert(GEMM_BK == 64, "the pipeline below is written out for four sub-steps per K-step");
-    // wave-uniform: does any element of this wave's sub-tile lie inside the matrices?
-    const bool live = __builtin_amdgcn_readfirstlane(
-        (A.origin + wm * WM < A.ext) && (B_DUAL || B.origin + wn * WN < B.ext));
-    if (nfull > 0) {
-        typedef MmaPipe<T, BM, BN, WM, WN, A_MN, B_MN> Pipe;
-        typedef TileLoader<T, BM, NW, A_MN, false> LoadA;
-        typedef typename std::conditional<(B_MN && B_DUAL), TileLoaderV<T, BN, NW, B_MN, B_DUAL>,
-                                          TileLoader<T, BN, NW, B_MN, B_DUAL>>::type LoadB;
-        constexpr int LD = LoadA::NI + LoadB::NI;            // load instructions per wave and K-step
-        constexpr int PER = (LD + Pipe::MFMAS - 1) / Pipe::MFMAS;
-        LoadA la;
-        LoadB lb;
-        la.init(A, wave, lane);
-        lb.init(B, wave, lane);
-        // instruction IDX of the next K-step into the stage at `buf` (K-steps are issued in order)
-        auto issue_one = [&](auto idx, T* buf) {
-            constexpr int IDX = decltype(idx)::value;
-            if constexpr (IDX < LoadA::NI) la.template issue<IDX>(buf, wave);
-            else if constexpr (IDX < LD) lb.template issue<IDX - LoadA::NI>(buf + BM * GEMM_BK, wave);
-        };
-        auto issue = [&](T* buf) { static_for<0, LD>([&](auto idx) { issue_one(idx, buf); }); };
-        typename Pipe::Slot f0, f1;
-        const int ra = wm * WM, rb = wn * WN;
-        // both buffers are free at the start of a tile: the first two K-steps go out together and
-        // only the first is waited for (short-K tiles spend a visible share of their time here)
-        issue(smem);
-        if (nfull > 1) {
-            issue(smem + BUF);
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LD) : "memory");
-        } else {
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        }
-        __syncthreads();
-        if (!live) {
-            // no row (or column) of this wave's sub-tile exists: it keeps loading its share of the
-            // stages and meets every barrier of the loop below, and leaves the matrix cores of its
-            // SIMD to the wave it shares them with (the last row tile of an expert is mostly this)
-            for (int kt = 0; kt + 1 < nfull; ++kt) {
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-                __syncthreads();
-                if (kt + 2 < nfull) issue(smem + (kt & 1) * BUF);
-            }
-        } else {
-        Pipe::fetch_all(f0, smem, smem + BM * GEMM_BK, 0, ra, rb, lane);
-        for (int kt = 0; kt + 1 < nfull; ++kt) {
-            T* cur = smem + (kt & 1) * BUF;
-            T* nxt = smem + ((kt + 1) & 1) * BUF;
-            T* curb = cur + BM * GEMM_BK;
-            Pipe::template sub<true>(acc, f0, f1, cur, curb, 1, ra, rb, lane);
-            Pipe::template sub<true>(acc, f1, f0, cur, curb, 2, ra, rb, lane);
-            Pipe::template sub<true>(acc, f0, f1, cur, curb, 3, ra, rb, lane);
-            // Every read of `cur` has been issued.  Once they and this wave's loads of step kt+1 have
-            // landed, the barrier makes `nxt` readable and `cur` writable for everyone; the MFMAs of
-            // the last sub-step then run while the first fragments of step kt+1 are read and the
-            // loads of step kt+2 are issued into `cur`, PER of them after each MFMA (measured 2-3 %
-            // faster in every layout than issuing them in one burst after the barrier).
-            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-            __syncthreads();
-            const bool more = kt + 2 < nfull;
-            Pipe::template sub<true>(acc, f1, f0, nxt, nxt + BM * GEMM_BK, 0, ra, rb, lane, [&](auto m) {
-                constexpr int M = decltype(m)::value;
-                if (more) static_for<M * PER, (M + 1) * PER>([&](auto idx) { issue_one(idx, cur); });
-            });
-        }
-        {   // last full K-step: nothing follows it in these buffers
-            T* cur = smem + ((nfull - 1) & 1) * BUF;
-            T* curb = cur + BM * GEMM_BK;
-            Pipe::template sub<true>(acc, f0, f1, cur, curb, 1, ra, rb, lane);
-            Pipe::template sub<true>(acc, f1, f0, cur, curb, 2, ra, rb, lane);
-            Pipe::template sub<true>(acc, f0, f1, cur, curb, 3, ra, rb, lane);
-            Pipe::template sub<false>(acc, f1, f0, cur, curb, 0, ra, rb, lane);
-        }
-        }
-    }
-    if (!B_DUAL && nfull * GEMM_BK < K) {  // K tail: through registers into the K-contiguous layout, zero-filled past K
-        Staged2<BM, NT> sa;
-        Staged2<BN, NT> sb;
-        T* buf = smem + (nfull & 1) * BUF;
-        stage2_load<T, BM, NT, A_MN>(sa, A, nfull * GEMM_BK, K, tid);
-        stage2_load<T, BN, NT, B_MN>(sb, B, nfull * GEMM_BK, K, tid);
-        stage2_store<T, BM, NT, A_MN>(sa, buf, tid);     // `buf` was last read two steps ago
-        stage2_store<T, BN, NT, B_MN>(sb, buf + BM * GEMM_BK, tid);
-        __syncthreads();
-        if (live) mma_step<T, BM, BN, WM, WN, false, false>(buf, buf + BM * GEMM_BK, wm * WM, wn * WN, lane, acc);
-    }
-    __syncthreads();  // every wave is past its last LDS read: the buffers become epilogue staging
+    MainLoop2<T, BM, BN, WAVES_M, WAVES_N, A_MN, B_MN, B_DUAL, ZERO> loop;
+    loop.begin(A, B, K, smem);
+    loop.finish(A, B, K, smem, smem + loop.BUF, acc);
     static_assert(gemm2_lds_bytes<T, BM, BN, WAVES_M, WAVES_N>() <= 160 * 1024, "tile configuration exceeds the 160 KB of LDS");
 }
 
@@ -739,14 +781,16 @@ struct Tile32Loader {
         half = op.half;
         if (!MN) {
             const int rr = lane >> 2, pos = lane & 3;
+            const bool gathered = !DUAL && op.row_map != nullptr;      // wave-uniform (see TileLoader)
 #pragma unroll
             for (int j = 0; j < NI; ++j) {
                 const int r = (j * NW + wave) * 16 + rr;
                 int g = op.origin + (DUAL ? op.dual_index(r) : r);
                 g = g < op.ext ? g : op.ext - 1;
-                off[j] = (unsigned)(((int64_t)(g - op.origin) * op.ld + (pos ^ swz_k<32>(r)) * 8) * (int64_t)sizeof(T));
+                const int64_t row = gathered ? (int64_t)op.row_map[g] : (int64_t)(g - op.origin);
+                off[j] = (unsigned)((row * op.ld + (pos ^ swz_k<32>(r)) * 8) * (int64_t)sizeof(T));
             }
-            base = op.base + (int64_t)op.origin * op.ld;
+            base = gathered ? op.base : op.base + (int64_t)op.origin * op.ld;
             base2 = DUAL ? op.base2 + (int64_t)op.origin * op.ld : nullptr;
             step = 32;
         } else {

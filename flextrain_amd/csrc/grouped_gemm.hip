@@ -133,7 +133,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64, K32 ? 2 : 1) void grouped_r
     const T* __restrict__ A, int64_t lda, const T* __restrict__ B, int64_t ldb, int64_t b_expert_stride,
     int64_t b2_delta, T* P1, T* P2, int64_t ldp, T* ACTO, int64_t ldact, const int32_t* __restrict__ NTILES,
     const int32_t* __restrict__ OFFSETS, const int32_t* __restrict__ TILES, int Nh, int K, int gate_first,
-    int tiles_n) {
+    int tiles_n, const int32_t* __restrict__ A_ROW_MAP) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T* smem = reinterpret_cast<T*>(smem_raw);
     const int total = NTILES[0] * tiles_n;
@@ -145,7 +145,10 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64, K32 ? 2 : 1) void grouped_r
     const int m0 = TILES[2 * tile + 1];
     const int64_t row0 = OFFSETS[e];
     const int rows = OFFSETS[e + 1] - OFFSETS[e];
-    OperandView<T> a{A + row0 * lda, lda, rows, m0};
+    // A_ROW_MAP: expert-sorted row r is row A_ROW_MAP[r] of A (the token it was routed from): the
+    // rows are gathered by the tile loads themselves and no expert-sorted copy of A exists
+    OperandView<T> a{A_ROW_MAP ? A : A + row0 * lda, lda, rows, m0};
+    if (A_ROW_MAP) a.row_map = A_ROW_MAP + row0;
     const T* b1 = B + (int64_t)e * b_expert_stride;
     OperandView<T> b{b1, ldb, Nh, tn * (BN / 2), BN / WAVES_N / 2, b1 + b2_delta};
     gemm_tile2_glu<T, BM, BN, WAVES_M, WAVES_N, B_MN, ACT_SILU, K32>(a, b, P1 + row0 * ldp, P2 + row0 * ldp, ldp,
@@ -153,24 +156,132 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64, K32 ? 2 : 1) void grouped_r
                                                                      gate_first != 0, smem);
 }
 
-template <typename T, typename TG, int BM, int BN, int WAVES_M, int WAVES_N>
-__global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void grouped_wgrad_kernel(
-    const T* __restrict__ A, int64_t lda, const T* __restrict__ B, int64_t ldb, TG* G, int64_t ldg,
-    int64_t g_expert_stride, const int32_t* __restrict__ OFFSETS, int M, int N, float alpha, float beta,
-    int tiles_n, int tiles_per_expert) {
+// ---------------------------------------------------------------- workgroups that walk several tiles
+// One workgroup per CU walks the tile list with a stride of the grid size.  Between the K loop of a
+// tile and its epilogue it sets up the next tile's loaders and requests that tile's first K-step,
+// so the cold start of a tile (table look-ups, first loads: 2-3 us of a 25-70 us tile) runs under
+// the epilogue of the one before.  LDS plan (160 KB): [stage 0: 64 KB][32 KB][stage 1: 64 KB]; the
+// epilogue stages its bands in the 96 KB behind stage 0, which only the SECOND K-step of the next
+// tile overwrites, and that is issued after the barrier that follows the epilogue.
+constexpr size_t kWalkLdsBytes = 160 * 1024;
+
+template <typename T>
+struct WalkLds {
+    static FX_DEV T* buf0(T* smem) { return smem; }
+    static FX_DEV T* epi(T* smem) { return smem + 64 * 1024 / sizeof(T); }
+    static FX_DEV T* buf1(T* smem) { return smem + 96 * 1024 / sizeof(T); }
+};
+
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool B_MN>
+__global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void grouped_rows_walk_kernel(
+    const T* __restrict__ A, int64_t lda, const T* __restrict__ B, int64_t ldb, int64_t b_expert_stride,
+    const T* C, int64_t ldc, T* D, int64_t ldd, const int32_t* __restrict__ NTILES,
+    const int32_t* __restrict__ OFFSETS, const int32_t* __restrict__ TILES, int N, int K, float alpha,
+    float beta, int tiles_n) {
+    static_assert((BM + BN) * GEMM_BK * sizeof(T) == 64 * 1024, "the LDS plan assumes 64 KB stages");
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T* smem = reinterpret_cast<T*>(smem_raw);
-    // expert-major tile order, one contiguous band of it per XCD (see grouped_rows_kernel)
-    const int p = xcd_band(blockIdx.x, gridDim.x);
-    const int e = p / tiles_per_expert, t = p % tiles_per_expert;
-    const int64_t row0 = OFFSETS[e];
-    const int rows = OFFSETS[e + 1] - OFFSETS[e];
-    if (rows == 0 && beta == 1.f) return;  // nothing to add
-    const int tm = t / tiles_n, tn = t % tiles_n;
-    OperandView<T> a{A + row0 * lda, lda, M, tm * BM};
-    OperandView<T> b{B + row0 * ldb, ldb, N, tn * BN};
-    TG* g = G + (int64_t)e * g_expert_stride;
-    gemm_tile2<T, TG, BM, BN, WAVES_M, WAVES_N, true, true>(a, b, g, g, ldg, ldg, M, N, rows, alpha, beta, smem);
+    constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+    const int total = NTILES[0] * tiles_n;
+    int pid = blockIdx.x;
+    if (pid >= total) return;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    struct Tile { int m0, tn, rows, e; int64_t row0; };
+    auto lookup = [&](int id) {
+        const int p = xcd_band(id, total);
+        const int tile = p / tiles_n;
+        Tile t;
+        t.tn = p % tiles_n;
+        t.e = TILES[2 * tile];
+        t.m0 = TILES[2 * tile + 1];
+        t.row0 = OFFSETS[t.e];
+        t.rows = OFFSETS[t.e + 1] - OFFSETS[t.e];
+        return t;
+    };
+    auto view_a = [&](const Tile& t) { return OperandView<T>{A + t.row0 * lda, lda, t.rows, t.m0}; };
+    auto view_b = [&](const Tile& t) { return OperandView<T>{B + (int64_t)t.e * b_expert_stride, ldb, N, t.tn * BN}; };
+    MainLoop2<T, BM, BN, WAVES_M, WAVES_N, false, B_MN> loop;
+    Tile cur = lookup(pid);
+    OperandView<T> a = view_a(cur), b = view_b(cur);
+    loop.begin(a, b, K, WalkLds<T>::buf0(smem));
+    bool landed = false;     // from the second tile on, K-step 0 has landed and been published by the epilogue's wait + barrier
+    for (;;) {
+        const int npid = pid + (int)gridDim.x;
+        const bool more = npid < total;
+        Tile nxt = cur;
+        if (more) nxt = lookup(npid);
+        f32x16_t acc[WM / 32][WN / 32];
+        loop.finish(a, b, K, WalkLds<T>::buf0(smem), WalkLds<T>::buf1(smem), acc, landed);
+        const OperandView<T> a2 = view_a(nxt), b2 = view_b(nxt);
+        if (more) loop.begin(a2, b2, K, WalkLds<T>::buf0(smem));
+        epilogue_tile<T, T, WM, WN, true>(acc, C ? C + cur.row0 * ldc : nullptr, D + cur.row0 * ldd, ldc, ldd,
+                                    cur.m0 + (wave / WAVES_N) * WM, cur.tn * BN + (wave % WAVES_N) * WN, cur.rows, N, alpha,
+                                    beta, WalkLds<T>::epi(smem), wave, lane);
+        if (!more) break;
+        __syncthreads();     // every wave is done with its staging area before stage 1 is written again
+        landed = true;
+        cur = nxt;
+        a = a2;
+        b = b2;
+        pid = npid;
+    }
+}
+
+template <typename T, typename TG, int BM, int BN, int WAVES_M, int WAVES_N>
+__global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void grouped_wgrad_walk_kernel(
+    const T* __restrict__ A, int64_t lda, const T* __restrict__ B, int64_t ldb, TG* G, int64_t ldg,
+    int64_t g_expert_stride, const int32_t* __restrict__ OFFSETS, int M, int N, float alpha, float beta,
+    int tiles_n, int tiles_per_expert, int total) {
+    static_assert((BM + BN) * GEMM_BK * sizeof(T) == 64 * 1024, "the LDS plan assumes 64 KB stages");
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T* smem = reinterpret_cast<T*>(smem_raw);
+    constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+    int pid = blockIdx.x;
+    if (pid >= total) return;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    struct Tile { int e, tm, tn, rows; int64_t row0; };
+    auto lookup = [&](int id) {
+        const int p = xcd_band(id, total);
+        Tile t;
+        t.e = p / tiles_per_expert;
+        const int q = p % tiles_per_expert;
+        t.tm = q / tiles_n;
+        t.tn = q % tiles_n;
+        t.row0 = OFFSETS[t.e];
+        t.rows = OFFSETS[t.e + 1] - OFFSETS[t.e];
+        return t;
+    };
+    auto view_a = [&](const Tile& t) { return OperandView<T>{A + t.row0 * lda, lda, M, t.tm * BM}; };
+    auto view_b = [&](const Tile& t) { return OperandView<T>{B + t.row0 * ldb, ldb, N, t.tn * BN}; };
+    MainLoop2<T, BM, BN, WAVES_M, WAVES_N, true, true> loop;
+    Tile cur = lookup(pid);
+    OperandView<T> a = view_a(cur), b = view_b(cur);
+    loop.begin(a, b, cur.rows, WalkLds<T>::buf0(smem));
+    bool landed = false;
+    for (;;) {
+        const int npid = pid + (int)gridDim.x;
+        const bool more = npid < total;
+        Tile nxt = cur;
+        if (more) nxt = lookup(npid);
+        f32x16_t acc[WM / 32][WN / 32];
+        loop.finish(a, b, cur.rows, WalkLds<T>::buf0(smem), WalkLds<T>::buf1(smem), acc, landed);
+        const OperandView<T> a2 = view_a(nxt), b2 = view_b(nxt);
+        if (more) loop.begin(a2, b2, nxt.rows, WalkLds<T>::buf0(smem));
+        if (!(cur.rows == 0 && beta == 1.f)) {   // an expert without rows adds nothing
+            TG* g = G + (int64_t)cur.e * g_expert_stride;
+            epilogue_tile<T, TG, WM, WN, true>(acc, g, g, ldg, ldg, cur.tm * BM + (wave / WAVES_N) * WM,
+                                               cur.tn * BN + (wave % WAVES_N) * WN, M, N, alpha, beta, WalkLds<T>::epi(smem), wave, lane);
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the wait the skipped epilogue would have made
+        }
+        if (!more) break;
+        __syncthreads();
+        landed = true;
+        cur = nxt;
+        a = a2;
+        b = b2;
+        pid = npid;
+    }
 }
 
 static inline int cdiv_i(int64_t a, int b) { return (int)((a + b - 1) / b); }
@@ -178,6 +289,20 @@ static inline int cdiv_i(int64_t a, int b) { return (int)((a + b - 1) / b); }
 }  // namespace fx
 
 using namespace fx;
+
+// Workgroups of the walking kernels: one per CU of the current device.
+static int walk_grid() {
+    static int cus[64] = {};
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    if (dev < 0 || dev >= 64) return 256;
+    if (cus[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cus[dev] = (n / 8) * 8 > 0 ? (n / 8) * 8 : n;      // a multiple of the 8 XCDs keeps a workgroup's tiles on one XCD
+    }
+    return cus[dev];
+}
 
 extern "C" size_t fx_grouped_ws_bytes(int E, int64_t total_rows) {
     if (E <= 0 || total_rows < 0) return 0;
@@ -241,8 +366,20 @@ extern "C" int fx_grouped_gemm_rows(const void* A, int64_t lda, const void* B, i
         FX_CHECK_LAUNCH("fx_grouped_gemm_rows");
         return 0;
     }
+#define FX_ROWS_WALK(TT, BMN)                                                                             \
+    {                                                                                                     \
+        auto kern = grouped_rows_walk_kernel<TT, 256, 256, 2, 4, BMN>;                                    \
+        FX_ENSURE_DYNAMIC_LDS(kern, kWalkLdsBytes);                                                       \
+        const int tiles_n = cdiv_i(N, 256);                                                               \
+        const unsigned most = max_tiles * (unsigned)tiles_n;                                              \
+        const unsigned grid = most < (unsigned)walk_grid() ? most : (unsigned)walk_grid();                \
+        kern<<<dim3(grid), 512, kWalkLdsBytes, stream>>>(                                                 \
+            reinterpret_cast<const TT*>(A), lda, reinterpret_cast<const TT*>(B), ldb, b_expert_stride,    \
+            reinterpret_cast<const TT*>(C), ldc, reinterpret_cast<TT*>(D), ldd, w.ntiles, w.offsets,      \
+            w.tiles, N, K, alpha, beta, tiles_n);                                                         \
+    }
 #define FX_ROWS_T(TT)                                                                                     \
-    if (BM == 256) { if (trans_b) FX_ROWS(TT, 256, 256, 2, 4, false) else FX_ROWS(TT, 256, 256, 2, 4, true) } \
+    if (BM == 256) { if (trans_b) FX_ROWS_WALK(TT, false) else FX_ROWS_WALK(TT, true) }                   \
     else { if (trans_b) FX_ROWS(TT, 128, 128, 2, 2, false) else FX_ROWS(TT, 128, 128, 2, 2, true) }
     if (dt == DT_BF16) { FX_ROWS_T(bf16) } else { FX_ROWS_T(f16) }
 #undef FX_ROWS_T
@@ -254,7 +391,8 @@ extern "C" int fx_grouped_gemm_rows(const void* A, int64_t lda, const void* B, i
 extern "C" int fx_grouped_gemm_rows_glu(const void* A, int64_t lda, const void* B, int64_t ldb, int64_t b_expert_stride,
                                         int trans_b, int64_t b2_delta, void* P1, void* P2, int64_t ldp, void* act,
                                         int64_t ldact, const int32_t* counts, int E, int64_t total_rows, int Nh, int K,
-                                        int gate_first, int dt, void* ws, size_t ws_bytes, hipStream_t stream) {
+                                        int gate_first, int dt, void* ws, size_t ws_bytes, const int32_t* a_row_map,
+                                        int64_t a_rows, hipStream_t stream) {
     if (E <= 0 || total_rows < 0 || Nh <= 0 || K <= 0) FX_FAIL("fx_grouped_gemm_rows_glu: bad shape");
     if (total_rows == 0) return 0;
     if (!A || !B || !P1 || !P2 || !act || !counts) FX_FAIL("fx_grouped_gemm_rows_glu: null pointer");
@@ -264,6 +402,8 @@ extern "C" int fx_grouped_gemm_rows_glu(const void* A, int64_t lda, const void* 
     if (!aligned16(A) || !aligned16(B) || !aligned16(P1) || !aligned16(P2) || !aligned16(act) || (lda & 7) || (ldb & 7) ||
         (ldp & 7) || (ldact & 7) || (K & 63) || (Nh & 7) || (b_expert_stride & 7) || (b2_delta & 7))
         FX_FAIL("fx_grouped_gemm_rows_glu: needs K %% 64 == 0, N %% 8 == 0, strides %% 8 == 0 and 16-byte aligned operands");
+    if (a_row_map && (a_rows <= 0 || (uint64_t)a_rows * (uint64_t)lda * 2u >= (1ull << 32)))
+        FX_FAIL("fx_grouped_gemm_rows_glu: a gathered A must have a_rows > 0 and stay below 4 GB");
     GroupedWs w = split_ws(ws, E);
     const int BM = rows_bm(total_rows, E);
     grouped_plan_kernel<<<1, 256, 0, stream>>>(counts, E, BM, w.ntiles, w.offsets, w.tiles);
@@ -278,7 +418,7 @@ extern "C" int fx_grouped_gemm_rows_glu(const void* A, int64_t lda, const void* 
         kern<<<dim3(max_tiles * (unsigned)tiles_n), WM_ * WN_ * 64, lds, stream>>>(                       \
             reinterpret_cast<const TT*>(A), lda, reinterpret_cast<const TT*>(B), ldb, b_expert_stride,    \
             b2_delta, reinterpret_cast<TT*>(P1), reinterpret_cast<TT*>(P2), ldp, reinterpret_cast<TT*>(act), \
-            ldact, w.ntiles, w.offsets, w.tiles, Nh, K, gate_first, tiles_n);                             \
+            ldact, w.ntiles, w.offsets, w.tiles, Nh, K, gate_first, tiles_n, a_row_map);                  \
     }
     // 128-row tiles: 128 x 256 (128 columns of each half) with 32-wide K-steps, two workgroups per CU
 #define FX_GLU_T(TT)                                                                                      \
@@ -309,19 +449,19 @@ extern "C" int fx_grouped_gemm_wgrad(const void* A, int64_t lda, const void* B, 
     constexpr int BM = 256, BN = 256;
     const int tiles_m = cdiv_i(M, BM), tiles_n = cdiv_i(N, BN);
     const dim3 grid((unsigned)(tiles_m * tiles_n) * (unsigned)E);
-#define FX_WG(TT, TG)                                                                                     \
+#define FX_WG_WALK(TT, TG)                                                                                \
     {                                                                                                     \
-        auto kern = grouped_wgrad_kernel<TT, TG, BM, BN, 2, 4>;                                           \
-        constexpr size_t lds = gemm2_lds_bytes<TT, BM, BN, 2, 4>();                                       \
-        FX_ENSURE_DYNAMIC_LDS(kern, lds);                                                                 \
-        kern<<<grid, 2 * 4 * 64, lds, stream>>>(reinterpret_cast<const TT*>(A), lda,                      \
-                                                reinterpret_cast<const TT*>(B), ldb, reinterpret_cast<TG*>(G), \
-                                                ldg, g_expert_stride, w.offsets, M, N, alpha, beta, tiles_n, tiles_m * tiles_n); \
+        auto kern = grouped_wgrad_walk_kernel<TT, TG, BM, BN, 2, 4>;                                      \
+        FX_ENSURE_DYNAMIC_LDS(kern, kWalkLdsBytes);                                                       \
+        const unsigned grid_w = grid.x < (unsigned)walk_grid() ? grid.x : (unsigned)walk_grid();          \
+        kern<<<dim3(grid_w), 2 * 4 * 64, kWalkLdsBytes, stream>>>(                                        \
+            reinterpret_cast<const TT*>(A), lda, reinterpret_cast<const TT*>(B), ldb, reinterpret_cast<TG*>(G), ldg, \
+            g_expert_stride, w.offsets, M, N, alpha, beta, tiles_n, tiles_m * tiles_n, (int)grid.x);      \
     }
-    if (dt == DT_BF16 && g_dt == DT_BF16) FX_WG(bf16, bf16)
-    else if (dt == DT_BF16) FX_WG(bf16, float)
-    else FX_WG(f16, f16)
-#undef FX_WG
+    if (dt == DT_BF16 && g_dt == DT_BF16) FX_WG_WALK(bf16, bf16)
+    else if (dt == DT_BF16) FX_WG_WALK(bf16, float)
+    else FX_WG_WALK(f16, f16)
+#undef FX_WG_WALK
     FX_CHECK_LAUNCH("fx_grouped_gemm_wgrad");
     return 0;
 }

@@ -252,6 +252,30 @@ extern "C" int fx_moe_scatter(const void* x, const void* indices, int indices_ar
     return 0;
 }
 
+// out[indices[t, k]] = t: the token each expert-sorted row was routed from.
+template <typename TI>
+__global__ __launch_bounds__(256) void moe_row_sources_kernel(const TI* __restrict__ IND, int64_t n, int K, int32_t* __restrict__ OUT) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const int64_t r = (int64_t)IND[i];
+    if (r >= 0 && r < n) OUT[r] = (int32_t)(i / K);
+}
+
+extern "C" int fx_moe_row_sources(const void* indices, int indices_are_int64, int64_t T, int K, int32_t* out,
+                                  hipStream_t stream) {
+    if (T < 0 || K <= 0) FX_FAIL("fx_moe_row_sources: bad shape");
+    if (T == 0) return 0;
+    if (!indices || !out) FX_FAIL("fx_moe_row_sources: null pointer");
+    const int64_t n = T * K;
+    const unsigned grid = (unsigned)((n + 255) / 256);
+    if (indices_are_int64)
+        moe_row_sources_kernel<int64_t><<<grid, 256, 0, stream>>>(reinterpret_cast<const int64_t*>(indices), n, K, out);
+    else
+        moe_row_sources_kernel<int32_t><<<grid, 256, 0, stream>>>(reinterpret_cast<const int32_t*>(indices), n, K, out);
+    FX_CHECK_LAUNCH("fx_moe_row_sources");
+    return 0;
+}
+
 extern "C" int fx_moe_scatter_weights(const void* weights, const void* indices, int indices_are_int64,
                                       void* out, int64_t n, int dt, hipStream_t stream) {
     if (n < 0) FX_FAIL("fx_moe_scatter_weights: negative count");

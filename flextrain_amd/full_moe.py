@@ -6,7 +6,8 @@ What differs underneath: the per-expert Python loop (one GEMM call per expert,
 alternating two streams, after a device->host copy of the counts and a stream
 synchronisation: full_moe.py:144-148, :428-466, :545-626) is replaced by
 grouped launches that read the counts on the device.  ``secondary_stream`` is
-accepted and left idle: one grouped launch already fills the GPU.
+accepted and left idle: one grouped launch already fills the GPU (measured both
+ways, see ``swiglu_expert_loop_bwd``).
 """
 from __future__ import annotations
 
@@ -26,6 +27,7 @@ from .ops.moe import (
     flextrain_load_balance_bwd,
     flextrain_moe_gather,
     flextrain_moe_router_gate_bwd,
+    flextrain_moe_row_sources,
     flextrain_moe_scatter,
     flextrain_moe_scatter_routing_weights,
     flextrain_moe_sort,
@@ -78,7 +80,8 @@ def dispatch_scatter(x, router_weights, topk_ids, *, num_experts, index_mapping,
     pinned = expert_counts_cpu if (expert_counts_cpu is not None and expert_counts_cpu.is_pinned()) else None
     indices, counts = flextrain_moe_sort(topk_ids, num_experts=num_experts, indices=index_mapping,
                                          expert_counts_gpu=expert_counts_gpu, expert_counts_pinned=pinned)
-    flextrain_moe_scatter(x, indices, out=scattered_x_out)
+    if scattered_x_out is not None:          # None: the caller's up-projection gathers the token rows itself
+        flextrain_moe_scatter(x, indices, out=scattered_x_out)
     flextrain_moe_scatter_routing_weights(router_weights, indices, out=scattered_router_weights_out)
     if expert_counts_cpu is not None and pinned is None:
         expert_counts_cpu.copy_(counts)  # pageable destination: synchronous copy (counts: the sort's own
@@ -95,11 +98,25 @@ def combine_gather(scattered_y, indices, *, router_weights, residual, out_tensor
 # ---------------------------------------------------------------------------
 # Expert compute (flextrain/ops/full_moe.py:393-679)
 # ---------------------------------------------------------------------------
+def gathered_up_projection_supported(x, w_up, x_preact_buf, expert_dim):
+    """Whether the expert up-projection can read the token rows of ``x`` in place through a row map
+    (the fused launch must take the operands, and ``x`` must stay below 4 GB)."""
+    TK = x_preact_buf.shape[0]
+    probe_act = torch.empty((0, expert_dim), dtype=x.dtype, device=x.device)
+    return (x.dim() == 2 and x.stride(1) == 1 and x.shape[0] * x.stride(0) * x.element_size() < (1 << 32)
+            and grouped_glu_supported(x, w_up, x_preact_buf[:TK], probe_act))
+
+
 def swiglu_expert_loop_fwd(scattered_x, x_preact_buf, w_up, w_down, expert_counts_cpu, *, primary_stream,
-                           secondary_stream=None, x_act_even=None, x_act_odd=None, expert_counts_gpu=None):
+                           secondary_stream=None, x_act_even=None, x_act_odd=None, expert_counts_gpu=None,
+                           gather_from=None, row_sources=None):
     """For every expert e over its rows: ``x_preact = x_e @ w_up[e].T`` (saved),
     ``act = silu(gate) * value``, ``scattered_x[rows] = act @ w_down[e].T``
-    (overwrites the input).  ``w_up (E, 2F, d)``, ``w_down (E, d, F)``."""
+    (overwrites the input).  ``w_up (E, 2F, d)``, ``w_down (E, d, F)``.
+
+    ``gather_from`` / ``row_sources`` (not in the reference): the unsorted ``(T, d)`` activations and
+    the token of every expert-sorted row; the up-projection then gathers its rows from
+    ``gather_from`` and ``scattered_x`` is only written (with the down-projection's result)."""
     TK = scattered_x.shape[0]
     F = w_down.shape[2]
     counts = _device_counts(expert_counts_cpu, expert_counts_gpu)
@@ -109,7 +126,9 @@ def swiglu_expert_loop_fwd(scattered_x, x_preact_buf, w_up, w_down, expert_count
             act = x_act_even[:TK]
         else:
             act = torch.empty((TK, F), dtype=scattered_x.dtype, device=scattered_x.device)
-        if grouped_glu_supported(scattered_x, w_up, pre, act):
+        if gather_from is not None:
+            flextrain_grouped_gemm_rows_glu(gather_from, w_up, counts, pre, act, row_sources=row_sources)
+        elif grouped_glu_supported(scattered_x, w_up, pre, act):
             flextrain_grouped_gemm_rows_glu(scattered_x, w_up, counts, pre, act)   # SwiGLU in the GEMM epilogue
         else:
             flextrain_grouped_gemm_rows(scattered_x, w_up.transpose(1, 2), counts, pre)
@@ -127,37 +146,20 @@ def swiglu_expert_loop_bwd(scattered_upstream, scattered_x, x_preact_buf, srw, d
     accumulator missing from ``grads`` (or None) is skipped."""
     TK = scattered_upstream.shape[0]
     counts = _device_counts(expert_counts_cpu, expert_counts_gpu)
-    two = secondary_stream is not None and secondary_stream != primary_stream
+    # One stream: every grouped launch fills all CUs with one resident workgroup each, so launches on a
+    # second stream only take CUs from the first (measured at 8192 tokens x 128 experts: weight
+    # gradients on the secondary stream 2.06 ms against 2.01 ms for the same work on one stream).
     with torch.cuda.stream(primary_stream):
         dx_act = torch.empty((TK, expert_dim), dtype=scattered_upstream.dtype, device=scattered_upstream.device)
         fwd_act = torch.empty_like(dx_act)
         flextrain_grouped_gemm_rows(scattered_upstream, w_down, counts, dx_act)                        # (a)
         flextrain_swiglu_moe_bwd(dx_act, x_preact_buf[:TK], srw[:TK], dx=dx_up_up_grouped[:TK], dw=dprobs[:TK],
                                  fwd_act=fwd_act)                                                       # (b)
-        if two:
-            ready = torch.cuda.Event()
-            ready.record(primary_stream)
-    # The two weight-gradient launches only read what (b) left behind and write the accumulators, so
-    # with a second stream they run beside the dgrad through w_up (the reference alternates its two
-    # streams between experts for the same reason, full_moe.py:420-466); the primary stream waits
-    # for them before this function returns, so every buffer is free for the caller as before.
-    wgrad_stream = secondary_stream if two else primary_stream
-    with torch.cuda.stream(wgrad_stream):
-        if two:
-            wgrad_stream.wait_event(ready)
         if grads.get("g_down") is not None:
             flextrain_grouped_gemm_wgrad(scattered_upstream, fwd_act, grads["g_down"], counts)          # (c)
-        if not two:
-            flextrain_grouped_gemm_rows(dx_up_up_grouped[:TK], w_up, counts, dx_pre_grouped[:TK])       # (d)
+        flextrain_grouped_gemm_rows(dx_up_up_grouped[:TK], w_up, counts, dx_pre_grouped[:TK])           # (d)
         if grads.get("g_up") is not None:
             flextrain_grouped_gemm_wgrad(dx_up_up_grouped[:TK], scattered_x, grads["g_up"], counts)     # (e)
-        if two:
-            done = torch.cuda.Event()
-            done.record(wgrad_stream)
-    if two:
-        with torch.cuda.stream(primary_stream):
-            flextrain_grouped_gemm_rows(dx_up_up_grouped[:TK], w_up, counts, dx_pre_grouped[:TK])       # (d)
-            primary_stream.wait_event(done)
 
 
 def swiglu_expert_loop_recompute_x_up(scattered_x, x_preact_buf, w_up, expert_counts_cpu, *, primary_stream,
@@ -238,4 +240,5 @@ __all__ = (
     "swiglu_expert_loop_fwd",
     "swiglu_expert_loop_bwd",
     "swiglu_expert_loop_recompute_x_up",
+    "gathered_up_projection_supported",
 )

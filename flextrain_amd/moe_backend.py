@@ -14,7 +14,7 @@ from typing import Any, Callable, Mapping, MutableMapping, Protocol, runtime_che
 import torch
 
 from . import full_moe
-from .ops.moe import flextrain_moe_gather, flextrain_moe_scatter
+from .ops.moe import flextrain_moe_gather, flextrain_moe_row_sources, flextrain_moe_scatter
 
 
 @dataclass(frozen=True)
@@ -100,15 +100,22 @@ class FlextrainMoEExpertCompute:
         host_counts = self._host_counts(chunk_extra, layer_id, num_experts)
         scattered_x = scratch_fn((TK, d_model), x.dtype)
         srw = slot.scattered_router_weights[:TK, :]
+        # When the fused up-projection can take the operands it reads the token rows of x in place
+        # through the row map, and the expert-sorted copy of x (one write and one read of TK x d) is
+        # never made; scattered_x then only receives the down-projection's result.
+        gathered = full_moe.gathered_up_projection_supported(x, weights["w_up"], slot.x_up[:TK], expert_dim)
         indices, _ = full_moe.dispatch_scatter(
             x, router_weights, chosen_experts, num_experts=num_experts, index_mapping=slot.index_mapping,
-            expert_counts_gpu=slot.expert_counts, expert_counts_cpu=host_counts, scattered_x_out=scattered_x,
+            expert_counts_gpu=slot.expert_counts, expert_counts_cpu=host_counts,
+            scattered_x_out=None if gathered else scattered_x,
             scattered_router_weights_out=srw, sync=False)   # nothing below reads the counts on the host
+        row_sources = flextrain_moe_row_sources(indices, out=scratch_fn((TK,), torch.int32)) if gathered else None
         x_act = scratch_fn((TK, expert_dim), x.dtype)
         full_moe.swiglu_expert_loop_fwd(
             scattered_x=scattered_x, x_preact_buf=slot.x_up, w_up=weights["w_up"], w_down=weights["w_down"],
             expert_counts_cpu=host_counts, primary_stream=primary_stream, secondary_stream=secondary_stream,
-            x_act_even=x_act, x_act_odd=x_act, expert_counts_gpu=slot.expert_counts)
+            x_act_even=x_act, x_act_odd=x_act, expert_counts_gpu=slot.expert_counts,
+            gather_from=x if gathered else None, row_sources=row_sources)
         full_moe.combine_gather(scattered_x, indices, router_weights=router_weights,
                                 residual=residual.view(-1, d_model) if residual is not None else None,
                                 out_tensor=out)

@@ -15,6 +15,7 @@ from .moe import (
     flextrain_fused_topk_softmax,
     flextrain_load_balance_bwd,
     flextrain_moe_gather,
+    flextrain_moe_row_sources,
     flextrain_moe_router_gate_bwd,
     flextrain_moe_scatter,
     flextrain_moe_scatter_routing_weights,
@@ -73,6 +74,7 @@ __all__ = [
     "flextrain_fused_topk_softmax",
     "flextrain_load_balance_bwd",
     "flextrain_moe_gather",
+    "flextrain_moe_row_sources",
     "flextrain_moe_router_gate_bwd",
     "flextrain_moe_scatter",
     "flextrain_moe_scatter_routing_weights",

@@ -101,25 +101,35 @@ def grouped_glu_supported(A, w_up, pre, act):
             and w_up.is_contiguous() and all(t.data_ptr() % 16 == 0 for t in (A, w_up, pre, act)))
 
 
-def flextrain_grouped_gemm_rows_glu(A, w_up, counts, pre, act):
+def flextrain_grouped_gemm_rows_glu(A, w_up, counts, pre, act, row_sources=None):
     """Expert up-projection and SwiGLU in one launch: ``pre[rows_e] = A[rows_e] @ w_up[e].T``
     (packed ``[value (F) | gate (F)]`` like ``w_up (E, 2F, K)``) and ``act = silu(gate) * value``,
-    the activation evaluated from the rounded ``pre`` as the separate kernel would."""
+    the activation evaluated from the rounded ``pre`` as the separate kernel would.
+
+    ``row_sources`` (int32, one entry per expert-sorted row, from ``flextrain_moe_row_sources``):
+    ``A`` is then the UNSORTED ``(T, K)`` activation matrix and sorted row ``r`` is
+    ``A[row_sources[r]]``, gathered by the kernel's own tile loads (no expert-sorted copy)."""
     _rowmajor(A, "A"), _rowmajor(pre, "pre"), _rowmajor(act, "act")
     if w_up.dim() != 3 or not w_up.is_contiguous():
         raise ValueError("w_up must be a contiguous (E, 2F, K) tensor")
     E, F2, K = w_up.shape
     F = F2 // 2
-    TK = A.shape[0]
+    TK = pre.shape[0]
     if A.shape[1] != K or tuple(pre.shape) != (TK, F2) or tuple(act.shape) != (TK, F):
         raise ValueError(f"shape mismatch: A {tuple(A.shape)}, w_up {tuple(w_up.shape)}, pre {tuple(pre.shape)}, "
                          f"act {tuple(act.shape)}")
+    if row_sources is None:
+        if A.shape[0] != TK:
+            raise ValueError(f"A has {A.shape[0]} rows, the outputs {TK}")
+    elif (row_sources.dtype != torch.int32 or row_sources.numel() != TK or not row_sources.is_contiguous()
+          or not row_sources.is_cuda):
+        raise ValueError(f"row_sources must be a contiguous int32 CUDA tensor with {TK} elements")
     ws, nbytes = _workspace(E, TK, A.device)
     es = pre.element_size()
     rc = lib().fx_grouped_gemm_rows_glu(ptr(A), A.stride(0), ptr(w_up), K, w_up.stride(0), 1, F * K, ptr(pre),
                                         pre.data_ptr() + F * es, pre.stride(0), ptr(act), act.stride(0),
                                         _counts_ptr(counts, E), E, TK, F, K, 0, dtype_enum(A.dtype), ptr(ws), nbytes,
-                                        stream_ptr(A.device))
+                                        ptr(row_sources), A.shape[0], stream_ptr(A.device))
     check(rc, "fx_grouped_gemm_rows_glu")
     return pre, act
 

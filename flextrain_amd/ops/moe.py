@@ -190,6 +190,25 @@ def flextrain_moe_scatter_routing_weights(weights, indices, out=None):
     return out
 
 
+def flextrain_moe_row_sources(indices, out=None):
+    """``out[indices[t, k]] = t``: the token each expert-sorted row was routed from (int32,
+    ``T*K`` entries).  No counterpart in the reference, which always scatters the activations into
+    an expert-sorted copy (flextrain/ops/full_moe.py:131-141); with this map the grouped
+    up-projection reads the token rows in place (``flextrain_grouped_gemm_rows_glu(row_sources=)``)."""
+    if not indices.is_cuda or indices.dim() != 2 or not indices.is_contiguous():
+        raise ValueError("indices must be a contiguous (T, K) CUDA tensor")
+    if indices.dtype not in (torch.int32, torch.int64):
+        raise ValueError("indices must be int32 or int64")
+    T, K = indices.shape
+    if out is None:
+        out = torch.empty(T * K, dtype=torch.int32, device=indices.device)
+    elif out.dtype != torch.int32 or out.numel() != T * K or not out.is_contiguous() or not out.is_cuda:
+        raise ValueError(f"out must be a contiguous int32 CUDA tensor with {T * K} elements")
+    rc = lib().fx_moe_row_sources(ptr(indices), _is64(indices), T, K, ptr(out), stream_ptr(indices.device))
+    check(rc, "fx_moe_row_sources")
+    return out
+
+
 def flextrain_moe_gather(expert_out, indices, weights=None, residual=None, out=None):
     """``out[t] = residual[t] + sum_k weights[t,k] * expert_out[indices[t,k]]``
     with an fp32 accumulator; flextrain/ops/_kernels/moe.py:1130-1271."""

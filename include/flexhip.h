@@ -191,6 +191,12 @@ int fx_moe_scatter(const void* x, const void* indices, int indices_are_int64, co
                    int scales_dt, void* out, int64_t T, int D, int K, int64_t out_row_stride, int dt,
                    hipStream_t stream);
 
+/* The token every expert-sorted row came from: out[indices[t, k]] = t for the (T, K) mapping that
+ * fx_moe_sort wrote (the inverse of flextrain/ops/_kernels/moe.py:649-834's index mapping, which the
+ * reference never needs because it always materialises the sorted copy).  out has T*K entries. */
+int fx_moe_row_sources(const void* indices, int indices_are_int64, int64_t T, int K, int32_t* out,
+                       hipStream_t stream);
+
 /* flextrain_moe_scatter_routing_weights (flextrain/ops/_kernels/moe.py:1053-1127). */
 int fx_moe_scatter_weights(const void* weights, const void* indices, int indices_are_int64, void* out,
                            int64_t n, int dt, hipStream_t stream);
@@ -271,11 +277,17 @@ int fx_grouped_gemm_wgrad(const void* A, int64_t lda, const void* B, int64_t ldb
  * B[e] holds two halves of Nh rows (trans_b = 1, (2*Nh, K) row-major) or Nh columns (trans_b = 0),
  * b2_delta elements apart.  P1 / P2 (row stride ldp) receive the two pre-activation halves,
  * act (rows, Nh) = silu(gate) * value with gate = P1 when gate_first else P2, computed from the
- * rounded P values.  Needs K % 64 == 0 and Nh % 8 == 0. */
+ * rounded P values.  Needs K % 64 == 0 and Nh % 8 == 0.
+ * a_row_map (optional, total_rows entries from fx_moe_row_sources): expert-sorted row r of the
+ * product is row a_row_map[r] of A, which then is the UNSORTED (a_rows, K) activation matrix: the
+ * tile loads gather the rows, and the scatter launch of flextrain/ops/full_moe.py:131-141 with its
+ * expert-sorted copy of the activations is not needed for this product.  a_rows * lda * 2 bytes
+ * must stay below 4 GB.  Without a map A is the expert-sorted (total_rows, K) matrix. */
 int fx_grouped_gemm_rows_glu(const void* A, int64_t lda, const void* B, int64_t ldb, int64_t b_expert_stride,
                              int trans_b, int64_t b2_delta, void* P1, void* P2, int64_t ldp, void* act,
                              int64_t ldact, const int32_t* counts, int E, int64_t total_rows, int Nh, int K,
-                             int gate_first, int dt, void* ws, size_t ws_bytes, hipStream_t stream);
+                             int gate_first, int dt, void* ws, size_t ws_bytes, const int32_t* a_row_map,
+                             int64_t a_rows, hipStream_t stream);
 
 /* Gate and up projections of the dense gated FFN with the activation in the epilogue: replaces the
  * two matmuls and the gated-activation launch of flextrain/nn/blocks/ffn_dense.py:130-146.

@@ -70,3 +70,32 @@ def test_grouped_glu_matches_separate_launches(dev, E, F, K, rows):
     ref_act = ops.flextrain_swiglu_moe_fwd(ref_pre)
     close(act, ref_act, what="act vs the separate kernel")
     close(act, o_glu.swiglu_fwd(ref_pre[:, F:].cpu(), ref_pre[:, :F].cpu()), what="act vs oracle")
+
+
+@pytest.mark.parametrize("T,topk,E,F,K", [(96, 2, 4, 96, 128),        # small experts: 128-row tiles, 32-wide K-steps
+                                          (2048, 4, 8, 384, 256),     # ~1024 rows per expert: 256-row tiles
+                                          (5, 1, 3, 8, 64)])
+def test_grouped_glu_gathers_token_rows_in_place(dev, T, topk, E, F, K):
+    """The up-projection reading the unsorted activations through the row map equals, bit for bit, the
+    same launch on the expert-sorted copy that flextrain_moe_scatter makes."""
+    g = gen(T * 3 + E + F)
+    x = randn(g, T, K).to(dev)
+    ids = torch.stack([torch.randperm(E, generator=g)[:topk] for _ in range(T)]).to(torch.int32).to(dev)
+    mapping, counts = ops.flextrain_moe_sort(ids, num_experts=E)
+    TK = T * topk
+    w_up = randn(g, E, 2 * F, K, std=K ** -0.5).to(dev)
+    sx = ops.flextrain_moe_scatter(x, mapping)
+    pre_ref, act_ref = torch.empty(TK, 2 * F, dtype=torch.bfloat16, device=dev), torch.empty(TK, F, dtype=torch.bfloat16, device=dev)
+    flextrain_grouped_gemm_rows_glu(sx, w_up, counts, pre_ref, act_ref)
+    src = ops.flextrain_moe_row_sources(mapping)
+    want_src = torch.empty(TK, dtype=torch.int32)
+    want_src[mapping.cpu().flatten().long()] = torch.arange(TK, dtype=torch.int32) // topk
+    assert torch.equal(src.cpu(), want_src)
+    pre, act = torch.full_like(pre_ref, 7.0), torch.full_like(act_ref, 7.0)
+    flextrain_grouped_gemm_rows_glu(x, w_up, counts, pre, act, row_sources=src)
+    assert torch.equal(pre, pre_ref) and torch.equal(act, act_ref)
+    with pytest.raises(ValueError):
+        flextrain_grouped_gemm_rows_glu(x, w_up, counts, pre, act, row_sources=src[:-1])
+    if topk > 1:
+        with pytest.raises(ValueError):
+            flextrain_grouped_gemm_rows_glu(x, w_up, counts, pre, act)      # T rows, TK outputs, no map
