@@ -252,6 +252,7 @@ extern "C" int fx_moe_scatter(const void* x, const void* indices, int indices_ar
     return 0;
 }
 
+namespace fx {
 // out[indices[t, k]] = t: the token each expert-sorted row was routed from.
 template <typename TI>
 __global__ __launch_bounds__(256) void moe_row_sources_kernel(const TI* __restrict__ IND, int64_t n, int K, int32_t* __restrict__ OUT) {
@@ -260,6 +261,7 @@ __global__ __launch_bounds__(256) void moe_row_sources_kernel(const TI* __restri
     const int64_t r = (int64_t)IND[i];
     if (r >= 0 && r < n) OUT[r] = (int32_t)(i / K);
 }
+}  // namespace fx
 
 extern "C" int fx_moe_row_sources(const void* indices, int indices_are_int64, int64_t T, int K, int32_t* out,
                                   hipStream_t stream) {
