@@ -301,7 +301,7 @@ struct TileLoader {
 
     FX_DEV void init(const OperandView<T>& op, int wave, int lane) {
         half = op.half;
-        if (!MN) {
+        if constexpr (!MN) {
             const int rr = lane >> 3, pos = lane & 7;
             const bool gathered = !DUAL && op.row_map != nullptr;      // wave-uniform
 #pragma unroll
@@ -895,6 +895,7 @@ FX_DEV void gemm_mainloop32(const OperandView<T>& A, const OperandView<T>& B, in
     __syncthreads();
     static_assert(gemm32_lds_bytes<T, BM, BN, WAVES_M, WAVES_N>() <= 80 * 1024, "two workgroups must fit the LDS of a CU");
 }
+
 
 // ---------------------------------------------------------------- workgroup -> tile maps
 // blockIdx.x -> (tile_m, tile_n).  Workgroups are dealt round-robin to the 8 XCDs,
