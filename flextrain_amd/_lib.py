@@ -66,6 +66,7 @@ _SIGNATURES = {
     "fx_moe_scatter": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int64, c_int, c_int,
                                c_int64, c_int, c_void_p]),
     "fx_moe_scatter_weights": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int, c_void_p]),
+    "fx_grouped_plan": (c_int, [c_void_p, c_int, c_int64, c_void_p, c_size_t, c_void_p]),
     "fx_moe_row_sources": (c_int, [c_void_p, c_int, c_int64, c_int, c_void_p, c_void_p]),
     "fx_moe_gather": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
                               c_int64, c_int, c_int, c_int, c_void_p]),

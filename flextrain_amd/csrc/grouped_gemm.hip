@@ -318,6 +318,16 @@ extern "C" size_t fx_grouped_ws_bytes(int E, int64_t total_rows) {
 // 128 x 128 with 64-wide ones.
 static int rows_bm(int64_t total_rows, int E) { return (total_rows / (E > 0 ? E : 1)) >= 384 ? 256 : 128; }
 
+extern "C" int fx_grouped_plan(const int32_t* counts, int E, int64_t total_rows, void* ws, size_t ws_bytes,
+                               hipStream_t stream) {
+    if (E <= 0 || total_rows < 0) FX_FAIL("fx_grouped_plan: bad shape");
+    if (!counts || !ws || ws_bytes < fx_grouped_ws_bytes(E, total_rows)) FX_FAIL("fx_grouped_plan: null pointer or workspace too small");
+    GroupedWs w = split_ws(ws, E);
+    grouped_plan_kernel<<<1, 256, 0, stream>>>(counts, E, rows_bm(total_rows, E), w.ntiles, w.offsets, w.tiles);
+    FX_CHECK_LAUNCH("fx_grouped_plan");
+    return 0;
+}
+
 extern "C" int fx_grouped_gemm_rows(const void* A, int64_t lda, const void* B, int64_t ldb,
                                     int64_t b_expert_stride, int trans_b, const void* C, int64_t ldc, void* D,
                                     int64_t ldd, const int32_t* counts, int E, int64_t total_rows, int N, int K,
@@ -325,7 +335,7 @@ extern "C" int fx_grouped_gemm_rows(const void* A, int64_t lda, const void* B, i
                                     hipStream_t stream) {
     if (E <= 0 || total_rows < 0 || N <= 0 || K <= 0) FX_FAIL("fx_grouped_gemm_rows: bad shape");
     if (total_rows == 0) return 0;
-    if (!A || !B || !D || !counts) FX_FAIL("fx_grouped_gemm_rows: null pointer");
+    if (!A || !B || !D) FX_FAIL("fx_grouped_gemm_rows: null pointer");
     if (!ws || ws_bytes < fx_grouped_ws_bytes(E, total_rows)) FX_FAIL("fx_grouped_gemm_rows: workspace too small");
     if (dt != DT_BF16 && dt != DT_F16) FX_FAIL("fx_grouped_gemm_rows: bf16 or fp16 only");
     if (lda >= (1 << 23) || ldb >= (1 << 23)) FX_FAIL("fx_grouped_gemm_rows: leading dimensions must be below 2^23 elements");
@@ -335,8 +345,10 @@ extern "C" int fx_grouped_gemm_rows(const void* A, int64_t lda, const void* B, i
     if (!C || beta == 0.f) { C = nullptr; beta = 0.f; }
     GroupedWs w = split_ws(ws, E);
     const int BM = rows_bm(total_rows, E);
-    grouped_plan_kernel<<<1, 256, 0, stream>>>(counts, E, BM, w.ntiles, w.offsets, w.tiles);
-    FX_CHECK_LAUNCH("fx_grouped_gemm_rows(plan)");
+    if (counts) {    // no counts: the workspace already holds the plan fx_grouped_plan made for them
+        grouped_plan_kernel<<<1, 256, 0, stream>>>(counts, E, BM, w.ntiles, w.offsets, w.tiles);
+        FX_CHECK_LAUNCH("fx_grouped_gemm_rows(plan)");
+    }
     const unsigned max_tiles = (unsigned)(total_rows / BM + E);
 #define FX_ROWS(TT, BM_, BN_, WM_, WN_, BMN)                                                              \
     {                                                                                                     \
@@ -395,7 +407,7 @@ extern "C" int fx_grouped_gemm_rows_glu(const void* A, int64_t lda, const void* 
                                         int64_t a_rows, hipStream_t stream) {
     if (E <= 0 || total_rows < 0 || Nh <= 0 || K <= 0) FX_FAIL("fx_grouped_gemm_rows_glu: bad shape");
     if (total_rows == 0) return 0;
-    if (!A || !B || !P1 || !P2 || !act || !counts) FX_FAIL("fx_grouped_gemm_rows_glu: null pointer");
+    if (!A || !B || !P1 || !P2 || !act) FX_FAIL("fx_grouped_gemm_rows_glu: null pointer");
     if (!ws || ws_bytes < fx_grouped_ws_bytes(E, total_rows)) FX_FAIL("fx_grouped_gemm_rows_glu: workspace too small");
     if (dt != DT_BF16 && dt != DT_F16) FX_FAIL("fx_grouped_gemm_rows_glu: bf16 or fp16 only");
     if (lda >= (1 << 23) || ldb >= (1 << 23)) FX_FAIL("fx_grouped_gemm_rows_glu: leading dimensions must be below 2^23 elements");
@@ -406,8 +418,10 @@ extern "C" int fx_grouped_gemm_rows_glu(const void* A, int64_t lda, const void* 
         FX_FAIL("fx_grouped_gemm_rows_glu: a gathered A must have a_rows > 0 and stay below 4 GB");
     GroupedWs w = split_ws(ws, E);
     const int BM = rows_bm(total_rows, E);
-    grouped_plan_kernel<<<1, 256, 0, stream>>>(counts, E, BM, w.ntiles, w.offsets, w.tiles);
-    FX_CHECK_LAUNCH("fx_grouped_gemm_rows_glu(plan)");
+    if (counts) {
+        grouped_plan_kernel<<<1, 256, 0, stream>>>(counts, E, BM, w.ntiles, w.offsets, w.tiles);
+        FX_CHECK_LAUNCH("fx_grouped_gemm_rows_glu(plan)");
+    }
     const unsigned max_tiles = (unsigned)(total_rows / BM + E);
 #define FX_GLU(TT, BM_, BN_, WM_, WN_, BMN, K32_)                                                         \
     {                                                                                                     \
@@ -436,7 +450,7 @@ extern "C" int fx_grouped_gemm_wgrad(const void* A, int64_t lda, const void* B, 
                                      int64_t total_rows, int M, int N, float alpha, float beta, int dt, void* ws,
                                      size_t ws_bytes, hipStream_t stream) {
     if (E <= 0 || total_rows < 0 || M <= 0 || N <= 0) FX_FAIL("fx_grouped_gemm_wgrad: bad shape");
-    if (!A || !B || !G || !counts) FX_FAIL("fx_grouped_gemm_wgrad: null pointer");
+    if (!A || !B || !G) FX_FAIL("fx_grouped_gemm_wgrad: null pointer");
     if (!ws || ws_bytes < fx_grouped_ws_bytes(E, total_rows)) FX_FAIL("fx_grouped_gemm_wgrad: workspace too small");
     if (dt != DT_BF16 && dt != DT_F16) FX_FAIL("fx_grouped_gemm_wgrad: bf16 or fp16 only");
     if (lda >= (1 << 23) || ldb >= (1 << 23)) FX_FAIL("fx_grouped_gemm_wgrad: leading dimensions must be below 2^23 elements");
@@ -444,8 +458,10 @@ extern "C" int fx_grouped_gemm_wgrad(const void* A, int64_t lda, const void* B, 
     if (!aligned16(A) || !aligned16(B) || (lda & 7) || (ldb & 7) || (M & 7) || (N & 7))
         FX_FAIL("fx_grouped_gemm_wgrad: operands must be 16-byte aligned with M and N multiples of 8");
     GroupedWs w = split_ws(ws, E);
-    grouped_plan_kernel<<<1, 256, 0, stream>>>(counts, E, 128, w.ntiles, w.offsets, w.tiles);
-    FX_CHECK_LAUNCH("fx_grouped_gemm_wgrad(plan)");
+    if (counts) {    // only the row offsets of the plan are used here: any tile height serves
+        grouped_plan_kernel<<<1, 256, 0, stream>>>(counts, E, 128, w.ntiles, w.offsets, w.tiles);
+        FX_CHECK_LAUNCH("fx_grouped_gemm_wgrad(plan)");
+    }
     constexpr int BM = 256, BN = 256;
     const int tiles_m = cdiv_i(M, BM), tiles_n = cdiv_i(N, BN);
     const dim3 grid((unsigned)(tiles_m * tiles_n) * (unsigned)E);

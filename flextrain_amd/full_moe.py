@@ -17,6 +17,7 @@ import torch
 
 from .matmul_dispatcher import CublasLtDispatcher
 from .ops.grouped import (
+    GroupedPlan,
     flextrain_grouped_gemm_rows,
     flextrain_grouped_gemm_rows_glu,
     flextrain_grouped_gemm_wgrad,
@@ -126,14 +127,15 @@ def swiglu_expert_loop_fwd(scattered_x, x_preact_buf, w_up, w_down, expert_count
             act = x_act_even[:TK]
         else:
             act = torch.empty((TK, F), dtype=scattered_x.dtype, device=scattered_x.device)
+        plan = GroupedPlan(counts, w_up.shape[0], TK, scattered_x.device)    # the counts are read once per pass
         if gather_from is not None:
-            flextrain_grouped_gemm_rows_glu(gather_from, w_up, counts, pre, act, row_sources=row_sources)
+            flextrain_grouped_gemm_rows_glu(gather_from, w_up, counts, pre, act, row_sources=row_sources, plan=plan)
         elif grouped_glu_supported(scattered_x, w_up, pre, act):
-            flextrain_grouped_gemm_rows_glu(scattered_x, w_up, counts, pre, act)   # SwiGLU in the GEMM epilogue
+            flextrain_grouped_gemm_rows_glu(scattered_x, w_up, counts, pre, act, plan=plan)   # SwiGLU in the GEMM epilogue
         else:
-            flextrain_grouped_gemm_rows(scattered_x, w_up.transpose(1, 2), counts, pre)
+            flextrain_grouped_gemm_rows(scattered_x, w_up.transpose(1, 2), counts, pre, plan=plan)
             flextrain_swiglu_moe_fwd(pre, out=act)
-        flextrain_grouped_gemm_rows(act, w_down.transpose(1, 2), counts, scattered_x)
+        flextrain_grouped_gemm_rows(act, w_down.transpose(1, 2), counts, scattered_x, plan=plan)
 
 
 def swiglu_expert_loop_bwd(scattered_upstream, scattered_x, x_preact_buf, srw, dprobs, w_up, w_down, grads,
@@ -152,14 +154,15 @@ def swiglu_expert_loop_bwd(scattered_upstream, scattered_x, x_preact_buf, srw, d
     with torch.cuda.stream(primary_stream):
         dx_act = torch.empty((TK, expert_dim), dtype=scattered_upstream.dtype, device=scattered_upstream.device)
         fwd_act = torch.empty_like(dx_act)
-        flextrain_grouped_gemm_rows(scattered_upstream, w_down, counts, dx_act)                        # (a)
+        plan = GroupedPlan(counts, w_up.shape[0], TK, scattered_upstream.device)
+        flextrain_grouped_gemm_rows(scattered_upstream, w_down, counts, dx_act, plan=plan)             # (a)
         flextrain_swiglu_moe_bwd(dx_act, x_preact_buf[:TK], srw[:TK], dx=dx_up_up_grouped[:TK], dw=dprobs[:TK],
                                  fwd_act=fwd_act)                                                       # (b)
         if grads.get("g_down") is not None:
-            flextrain_grouped_gemm_wgrad(scattered_upstream, fwd_act, grads["g_down"], counts)          # (c)
-        flextrain_grouped_gemm_rows(dx_up_up_grouped[:TK], w_up, counts, dx_pre_grouped[:TK])           # (d)
+            flextrain_grouped_gemm_wgrad(scattered_upstream, fwd_act, grads["g_down"], counts, plan=plan)   # (c)
+        flextrain_grouped_gemm_rows(dx_up_up_grouped[:TK], w_up, counts, dx_pre_grouped[:TK], plan=plan)    # (d)
         if grads.get("g_up") is not None:
-            flextrain_grouped_gemm_wgrad(dx_up_up_grouped[:TK], scattered_x, grads["g_up"], counts)     # (e)
+            flextrain_grouped_gemm_wgrad(dx_up_up_grouped[:TK], scattered_x, grads["g_up"], counts, plan=plan)  # (e)
 
 
 def swiglu_expert_loop_recompute_x_up(scattered_x, x_preact_buf, w_up, expert_counts_cpu, *, primary_stream,

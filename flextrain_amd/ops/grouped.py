@@ -23,12 +23,33 @@ def _workspace(E, total_rows, device):
     return torch.empty(nbytes // 4, dtype=torch.int32, device=device), nbytes
 
 
+class GroupedPlan:
+    """Row offsets and tile list of one routing (``fx_grouped_plan``), made once and passed as
+    ``plan=`` to several grouped launches of the same ``(counts, E, total_rows)``."""
+
+    def __init__(self, counts: torch.Tensor, E: int, total_rows: int, device):
+        self.E, self.total_rows = E, total_rows
+        self.ws, self.nbytes = _workspace(E, total_rows, device)
+        rc = lib().fx_grouped_plan(_counts_ptr(counts, E), E, total_rows, ptr(self.ws), self.nbytes, stream_ptr(device))
+        check(rc, "fx_grouped_plan")
+
+
+def _plan_or_workspace(plan, counts, E, total_rows, device):
+    """(counts pointer or None, workspace tensor, bytes): with a plan the counts are not read again."""
+    if plan is not None:
+        if plan.E != E or plan.total_rows != total_rows:
+            raise ValueError(f"the plan was made for E={plan.E}, rows={plan.total_rows}; this call has E={E}, rows={total_rows}")
+        return None, plan.ws, plan.nbytes
+    ws, nbytes = _workspace(E, total_rows, device)
+    return _counts_ptr(counts, E), ws, nbytes
+
+
 def _rowmajor(t, name):
     if t.dim() != 2 or t.stride(1) != 1:
         raise ValueError(f"{name} must be 2-D with unit column stride")
 
 
-def flextrain_grouped_gemm_rows(A, B, counts, D, C=None, alpha=1.0, beta=0.0):
+def flextrain_grouped_gemm_rows(A, B, counts, D, C=None, alpha=1.0, beta=0.0, plan=None):
     """``D[rows_e] = alpha * A[rows_e] @ B[e] + beta * C[rows_e]`` for every expert.
 
     ``A (TK, K)``, ``D``/``C (TK, N)`` are expert-sorted; ``B`` is ``(E, K, N)``
@@ -51,16 +72,16 @@ def flextrain_grouped_gemm_rows(A, B, counts, D, C=None, alpha=1.0, beta=0.0):
         raise TypeError("A, B, C, D must share a dtype")
     if C is not None:
         _rowmajor(C, "C")
-    ws, nbytes = _workspace(E, TK, A.device)
+    cptr, ws, nbytes = _plan_or_workspace(plan, counts, E, TK, A.device)
     rc = lib().fx_grouped_gemm_rows(ptr(A), A.stride(0), ptr(B), ldb, B.stride(0), trans_b, ptr(C),
                                     C.stride(0) if C is not None else 0, ptr(D), D.stride(0),
-                                    _counts_ptr(counts, E), E, TK, N, K, alpha, beta, dtype_enum(A.dtype),
+                                    cptr, E, TK, N, K, alpha, beta, dtype_enum(A.dtype),
                                     ptr(ws), nbytes, stream_ptr(A.device))
     check(rc, "fx_grouped_gemm_rows")
     return D
 
 
-def flextrain_grouped_gemm_wgrad(A, B, G, counts, alpha=1.0, beta=1.0):
+def flextrain_grouped_gemm_wgrad(A, B, G, counts, alpha=1.0, beta=1.0, plan=None):
     """``G[e] = alpha * A[rows_e].T @ B[rows_e] + beta * G[e]`` for every expert;
     ``A (TK, M)``, ``B (TK, N)`` expert-sorted, ``G (E, M, N)`` (bf16/fp16, or fp32
     for bf16 inputs)."""
@@ -73,9 +94,9 @@ def flextrain_grouped_gemm_wgrad(A, B, G, counts, alpha=1.0, beta=1.0):
         raise ValueError(f"shape mismatch: A {tuple(A.shape)}, B {tuple(B.shape)}, G {tuple(G.shape)}")
     if A.dtype != B.dtype:
         raise TypeError("A and B must share a dtype")
-    ws, nbytes = _workspace(E, TK, A.device)
+    cptr, ws, nbytes = _plan_or_workspace(plan, counts, E, TK, A.device)
     rc = lib().fx_grouped_gemm_wgrad(ptr(A), A.stride(0), ptr(B), B.stride(0), ptr(G), G.stride(1), G.stride(0),
-                                     dtype_enum(G.dtype), _counts_ptr(counts, E), E, TK, M, N, alpha, beta,
+                                     dtype_enum(G.dtype), cptr, E, TK, M, N, alpha, beta,
                                      dtype_enum(A.dtype), ptr(ws), nbytes, stream_ptr(A.device))
     check(rc, "fx_grouped_gemm_wgrad")
     return G
@@ -101,7 +122,7 @@ def grouped_glu_supported(A, w_up, pre, act):
             and w_up.is_contiguous() and all(t.data_ptr() % 16 == 0 for t in (A, w_up, pre, act)))
 
 
-def flextrain_grouped_gemm_rows_glu(A, w_up, counts, pre, act, row_sources=None):
+def flextrain_grouped_gemm_rows_glu(A, w_up, counts, pre, act, row_sources=None, plan=None):
     """Expert up-projection and SwiGLU in one launch: ``pre[rows_e] = A[rows_e] @ w_up[e].T``
     (packed ``[value (F) | gate (F)]`` like ``w_up (E, 2F, K)``) and ``act = silu(gate) * value``,
     the activation evaluated from the rounded ``pre`` as the separate kernel would.
@@ -124,11 +145,11 @@ def flextrain_grouped_gemm_rows_glu(A, w_up, counts, pre, act, row_sources=None)
     elif (row_sources.dtype != torch.int32 or row_sources.numel() != TK or not row_sources.is_contiguous()
           or not row_sources.is_cuda):
         raise ValueError(f"row_sources must be a contiguous int32 CUDA tensor with {TK} elements")
-    ws, nbytes = _workspace(E, TK, A.device)
+    cptr, ws, nbytes = _plan_or_workspace(plan, counts, E, TK, A.device)
     es = pre.element_size()
     rc = lib().fx_grouped_gemm_rows_glu(ptr(A), A.stride(0), ptr(w_up), K, w_up.stride(0), 1, F * K, ptr(pre),
                                         pre.data_ptr() + F * es, pre.stride(0), ptr(act), act.stride(0),
-                                        _counts_ptr(counts, E), E, TK, F, K, 0, dtype_enum(A.dtype), ptr(ws), nbytes,
+                                        cptr, E, TK, F, K, 0, dtype_enum(A.dtype), ptr(ws), nbytes,
                                         ptr(row_sources), A.shape[0], stream_ptr(A.device))
     check(rc, "fx_grouped_gemm_rows_glu")
     return pre, act

@@ -249,8 +249,15 @@ int fx_softmax_ce(const void* logits, void* dz_out, const void* labels, int labe
 
 /* ---- Expert-grouped GEMMs -------------------------------------------------- */
 
-/* Scratch bytes for the two grouped GEMM entry points (row offsets + tile list). */
+/* Scratch bytes for the grouped GEMM entry points (row offsets + tile list). */
 size_t fx_grouped_ws_bytes(int E, int64_t total_rows);
+
+/* Row offsets and tile list of one routing, made once and shared by several grouped launches: a
+ * grouped entry point called with counts == NULL takes the plan its workspace already holds (same E
+ * and total_rows) instead of making it again.  With the per-expert loop of
+ * flextrain/ops/full_moe.py:428-626 in mind: the counts are read once per pass over the experts,
+ * not once per GEMM. */
+int fx_grouped_plan(const int32_t* counts, int E, int64_t total_rows, void* ws, size_t ws_bytes, hipStream_t stream);
 
 /* The per-expert GEMMs of swiglu_expert_loop_fwd / _bwd / _recompute_x_up
  * (flextrain/ops/full_moe.py:428-466, :589-601, :613-616, :661-676) as one launch:

@@ -251,3 +251,33 @@ def test_recompute_and_phase_ops(dev):
                                     primary_stream=stream, secondary_stream=None,
                                     scratch_fn=lambda s, dt: torch.empty(s, dtype=dt, device=dev))
     assert torch.equal(handoff, saved) and torch.equal(slot.x_up, pre)
+
+
+@pytest.mark.parametrize("E,TK", [(8, 1000), (3, 5000)])
+def test_one_plan_serves_every_grouped_launch_of_a_routing(dev, E, TK):
+    """A GroupedPlan made once from the counts gives the same bits as each launch planning for itself."""
+    from flextrain_amd.ops.grouped import GroupedPlan, flextrain_grouped_gemm_rows_glu
+
+    g = gen(E + TK)
+    K, F = 128, 96
+    counts = _ragged_counts(g, E, TK).to(dev)
+    A = randn(g, TK, K, std=0.5).to(dev)
+    W = randn(g, E, 2 * F, K, std=0.1).to(dev)
+    Bw = randn(g, TK, 2 * F, std=0.5).to(dev)
+    plan = GroupedPlan(counts, E, TK, dev)
+    D0, D1 = (torch.full((TK, 2 * F), 7.0, dtype=torch.bfloat16, device=dev) for _ in range(2))
+    flextrain_grouped_gemm_rows(A, W.transpose(1, 2), counts, D0)
+    flextrain_grouped_gemm_rows(A, W.transpose(1, 2), None, D1, plan=plan)
+    assert torch.equal(D0, D1)
+    G0 = randn(g, E, K, 2 * F).to(dev)
+    G1 = G0.clone()
+    flextrain_grouped_gemm_wgrad(A, Bw, G0, counts)
+    flextrain_grouped_gemm_wgrad(A, Bw, G1, None, plan=plan)
+    assert torch.equal(G0, G1)
+    pre0, pre1 = torch.empty_like(D0), torch.empty_like(D0)
+    act0, act1 = (torch.empty(TK, F, dtype=torch.bfloat16, device=dev) for _ in range(2))
+    flextrain_grouped_gemm_rows_glu(A, W, counts, pre0, act0)
+    flextrain_grouped_gemm_rows_glu(A, W, None, pre1, act1, plan=plan)
+    assert torch.equal(pre0, pre1) and torch.equal(act0, act1)
+    with pytest.raises(ValueError):
+        flextrain_grouped_gemm_rows(A[:10], W.transpose(1, 2), None, D1[:10], plan=plan)
