@@ -25,7 +25,9 @@ def _workspace(E, total_rows, device):
 
 class GroupedPlan:
     """Row offsets and tile list of one routing (``fx_grouped_plan``), made once and passed as
-    ``plan=`` to several grouped launches of the same ``(counts, E, total_rows)``."""
+    ``plan=`` to several grouped launches of the same ``(counts, E, total_rows)``.  The plan is
+    written on the stream that is current when it is made: launches that use it must be ordered
+    after that point (same stream, or an event), and it must outlive them."""
 
     def __init__(self, counts: torch.Tensor, E: int, total_rows: int, device):
         self.E, self.total_rows = E, total_rows
@@ -40,6 +42,8 @@ def _plan_or_workspace(plan, counts, E, total_rows, device):
         if plan.E != E or plan.total_rows != total_rows:
             raise ValueError(f"the plan was made for E={plan.E}, rows={plan.total_rows}; this call has E={E}, rows={total_rows}")
         return None, plan.ws, plan.nbytes
+    if counts is None:
+        raise ValueError("expert counts are required when no plan is given")
     ws, nbytes = _workspace(E, total_rows, device)
     return _counts_ptr(counts, E), ws, nbytes
 
