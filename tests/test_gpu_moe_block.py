@@ -281,3 +281,34 @@ def test_one_plan_serves_every_grouped_launch_of_a_routing(dev, E, TK):
     assert torch.equal(pre0, pre1) and torch.equal(act0, act1)
     with pytest.raises(ValueError):
         flextrain_grouped_gemm_rows(A[:10], W.transpose(1, 2), None, D1[:10], plan=plan)
+
+
+def test_walking_kernels_fp16_and_int64_row_sources(dev):
+    """fp16 through the 256-row walking kernels (rows form and weight gradient), and the row map from an
+    int64 index mapping."""
+    from flextrain_amd.ops import moe as moe_ops
+
+    g = gen(4242)
+    E, TK, K, N = 3, 2400, 160, 264          # 800 rows per expert on average: 256-row tiles, K tail of 32
+    counts = _ragged_counts(g, E, TK)
+    A = randn(g, TK, K, std=0.5, dtype=torch.float16)
+    W = randn(g, E, N, K, std=0.1, dtype=torch.float16)
+    D = torch.empty(TK, N, dtype=torch.float16, device=dev)
+    flextrain_grouped_gemm_rows(A.to(dev), W.to(dev).transpose(1, 2), counts.to(dev), D)
+    off = o_moe.expert_offsets(counts)
+    for e in range(E):
+        a, b = int(off[e]), int(off[e + 1])
+        if a < b:
+            _close_scaled(D[a:b], A[a:b].float() @ W[e].float().t(), f"rows, expert {e}")
+    B = randn(g, TK, N, std=0.5, dtype=torch.float16)
+    G0 = randn(g, E, K, N, dtype=torch.float16)
+    G = G0.to(dev).clone()
+    flextrain_grouped_gemm_wgrad(A.to(dev), B.to(dev), G, counts.to(dev))
+    for e in range(E):
+        a, b = int(off[e]), int(off[e + 1])
+        _close_scaled(G[e], G0[e].float() + A[a:b].float().t() @ B[a:b].float(), f"wgrad, expert {e}")
+    ids = torch.stack([torch.randperm(8, generator=g)[:2] for _ in range(50)]).to(torch.int64).to(dev)
+    mapping, _ = moe_ops.flextrain_moe_sort(ids, num_experts=8)
+    src32 = moe_ops.flextrain_moe_row_sources(mapping.to(torch.int32))
+    src64 = moe_ops.flextrain_moe_row_sources(mapping.to(torch.int64))
+    assert torch.equal(src32, src64)
