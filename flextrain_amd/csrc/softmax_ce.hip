@@ -83,19 +83,29 @@ FX_DEV RowStat block_stat(RowStat s, float* sm_f, int* sm_i) {
     return r;
 }
 
+// Final-logit soft cap (flextrain/nn/head.py:273-282): y = cap * tanh(x / cap), rounded to the
+// storage type as the reference's in-place buffer is, so that argmax, maximum probability and loss
+// see the values a separate capping pass would have left in memory.
 template <typename T>
-FX_DEV RowStat row_sweep(const T* __restrict__ x, int V, float inv_temp, bool vec) {
+FX_DEV float softcap_value(float x, float cap, float inv_cap) {
+    return (float)(T)(cap * tanhf(x * inv_cap));
+}
+
+template <typename T, bool CAP = false>
+FX_DEV RowStat row_sweep(const T* __restrict__ x, int V, float inv_temp, bool vec, float cap = 0.f) {
     RowStat s{NEG_INF_F, 0.f, NEG_INF_F, 0x7fffffff};
+    const float inv_cap = CAP ? 1.0f / cap : 0.f;
     if (vec) {
         for (int c = threadIdx.x * 8; c < V; c += SM_THREADS * 8) {
             float v[8];
             load_f32<T, 8>(x + c, v);
 #pragma unroll
-            for (int j = 0; j < 8; ++j) v[j] *= inv_temp;
+            for (int j = 0; j < 8; ++j) v[j] = CAP ? softcap_value<T>(v[j], cap, inv_cap) : v[j] * inv_temp;
             stat_add_pack(s, v, c);
         }
     } else {
-        for (int c = threadIdx.x; c < V; c += SM_THREADS) stat_add(s, (float)x[c] * inv_temp, c);
+        for (int c = threadIdx.x; c < V; c += SM_THREADS)
+            stat_add(s, CAP ? softcap_value<T>((float)x[c], cap, inv_cap) : (float)x[c] * inv_temp, c);
     }
     return s;
 }
@@ -154,11 +164,13 @@ __global__ __launch_bounds__(256) void cross_entropy_kernel(T* __restrict__ P, c
 //   valid = 0 <= label < V
 //   loss  = keep && valid ? min(lse - x[label], max_loss) : 0
 //   dZ    = keep ? softmax(x) - (valid ? onehot(label) : 0) : 0
-template <typename T, typename TL>
+// CAP: the statistics, the loss and the probabilities are those of y = cap * tanh(x / cap), and dZ
+// is the gradient at x, i.e. multiplied by dy/dx = 1 - (y / cap)^2 (flextrain/nn/head.py:273-298).
+template <typename T, typename TL, bool CAP>
 __global__ __launch_bounds__(SM_THREADS) void softmax_ce_kernel(
     const T* X, T* DZ /* may alias X */, const TL* __restrict__ LABELS, const uint8_t* __restrict__ MASK,
     float* __restrict__ LOSS, int64_t* __restrict__ MAX_IDX, float* __restrict__ MAX_VAL, int V, int64_t in_stride,
-    int64_t out_stride, int64_t ignore_index, float max_loss, bool vec) {
+    int64_t out_stride, int64_t ignore_index, float max_loss, bool vec, float cap) {
     __shared__ float sm_f[3 * SM_THREADS / 64];
     __shared__ int sm_i[SM_THREADS / 64];
     const int64_t row = blockIdx.x;
@@ -167,13 +179,17 @@ __global__ __launch_bounds__(SM_THREADS) void softmax_ce_kernel(
     const int64_t label = (int64_t)LABELS[row];
     const bool keep = label != ignore_index && (MASK == nullptr || MASK[row] != 0);
     const bool valid = label >= 0 && label < V;
-    const RowStat st = block_stat(row_sweep<T>(x, V, 1.0f, vec), sm_f, sm_i);
+    const RowStat st = block_stat(row_sweep<T, CAP>(x, V, 1.0f, vec, cap), sm_f, sm_i);
     const float inv_l = 1.0f / st.l;
+    const float inv_cap = CAP ? 1.0f / cap : 0.f;
     if (threadIdx.x == 0) {
         if (MAX_IDX) MAX_IDX[row] = st.idx;
         if (MAX_VAL) MAX_VAL[row] = inv_l;
         float loss = 0.f;
-        if (keep && valid) loss = fminf((st.m + logf(st.l)) - (float)x[label], max_loss);
+        if (keep && valid) {
+            const float xl = CAP ? softcap_value<T>((float)x[label], cap, inv_cap) : (float)x[label];
+            loss = fminf((st.m + logf(st.l)) - xl, max_loss);
+        }
         LOSS[row] = loss;
     }
     __syncthreads();  // x[label] is read before any lane overwrites the row in place
@@ -185,8 +201,10 @@ __global__ __launch_bounds__(SM_THREADS) void softmax_ce_kernel(
                 load_f32<T, 8>(x + c, v);
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
-                    v[j] = __expf(v[j] - st.m) * inv_l;
+                    const float y = CAP ? softcap_value<T>(v[j], cap, inv_cap) : v[j];
+                    v[j] = __expf(y - st.m) * inv_l;
                     if (c + j == hot) v[j] -= 1.0f;
+                    if (CAP) v[j] *= 1.0f - (y * inv_cap) * (y * inv_cap);
                 }
             } else {
 #pragma unroll
@@ -198,10 +216,63 @@ __global__ __launch_bounds__(SM_THREADS) void softmax_ce_kernel(
         for (int c = threadIdx.x; c < V; c += SM_THREADS) {
             float v = 0.f;
             if (keep) {
-                v = __expf((float)x[c] - st.m) * inv_l;
+                const float y = CAP ? softcap_value<T>((float)x[c], cap, inv_cap) : (float)x[c];
+                v = __expf(y - st.m) * inv_l;
                 if (c == hot) v -= 1.0f;
+                if (CAP) v *= 1.0f - (y * inv_cap) * (y * inv_cap);
             }
             o[c] = (T)v;
+        }
+    }
+}
+
+// The soft cap as two passes of its own, for loss objects that are not the fused kernel above
+// (flextrain/nn/head.py:273-298): forward caps X in place and stores the gate 1 - (y / cap)^2,
+// computed from the rounded y, in the storage type; backward multiplies dZ by the gate.
+template <typename T>
+__global__ __launch_bounds__(256) void softcap_fwd_kernel(T* __restrict__ X, T* __restrict__ GATE, int64_t rows, int V,
+                                                          int64_t x_stride, int64_t g_stride, float cap, bool vec) {
+    const float inv_cap = 1.0f / cap;
+    const int per_row = vec ? V / 8 : V;
+    const int64_t total = rows * per_row;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const int64_t r = i / per_row;
+        const int c = (int)(i % per_row);
+        if (vec) {
+            float v[8], gt[8];
+            load_f32<T, 8>(X + r * x_stride + c * 8, v);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                v[j] = softcap_value<T>(v[j], cap, inv_cap);
+                gt[j] = 1.0f - (v[j] * inv_cap) * (v[j] * inv_cap);
+            }
+            store_f32<T, 8>(X + r * x_stride + c * 8, v);
+            store_f32<T, 8>(GATE + r * g_stride + c * 8, gt);
+        } else {
+            const float y = softcap_value<T>((float)X[r * x_stride + c], cap, inv_cap);
+            X[r * x_stride + c] = (T)y;
+            GATE[r * g_stride + c] = (T)(1.0f - (y * inv_cap) * (y * inv_cap));
+        }
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void softcap_bwd_kernel(T* __restrict__ DZ, const T* __restrict__ GATE, int64_t rows,
+                                                          int V, int64_t dz_stride, int64_t g_stride, bool vec) {
+    const int per_row = vec ? V / 8 : V;
+    const int64_t total = rows * per_row;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const int64_t r = i / per_row;
+        const int c = (int)(i % per_row);
+        if (vec) {
+            float v[8], gt[8];
+            load_f32<T, 8>(DZ + r * dz_stride + c * 8, v);
+            load_f32<T, 8>(GATE + r * g_stride + c * 8, gt);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] *= gt[j];
+            store_f32<T, 8>(DZ + r * dz_stride + c * 8, v);
+        } else {
+            DZ[r * dz_stride + c] = (T)((float)DZ[r * dz_stride + c] * (float)GATE[r * g_stride + c]);
         }
     }
 }
@@ -246,16 +317,53 @@ extern "C" int fx_cross_entropy(void* probs, const void* labels, int labels_are_
 extern "C" int fx_softmax_ce(const void* logits, void* dz_out, const void* labels, int labels_are_int64,
                              const uint8_t* loss_mask, float* loss_out, int64_t* max_idx_out, float* max_val_out,
                              int64_t rows, int V, int64_t in_row_stride, int64_t out_row_stride, int64_t ignore_index,
-                             float max_loss, int dt, hipStream_t stream) {
+                             float max_loss, float softcap, int dt, hipStream_t stream) {
     if (rows < 0 || V <= 0) FX_FAIL("fx_softmax_ce: bad shape");
+    if (!(softcap >= 0.f)) FX_FAIL("fx_softmax_ce: softcap must be 0 (off) or positive");
     if (rows == 0) return 0;
     if (!logits || !dz_out || !labels || !loss_out) FX_FAIL("fx_softmax_ce: null pointer");
     const bool vec = (V % 8 == 0) && (in_row_stride % 8 == 0) && (out_row_stride % 8 == 0) && aligned16(logits) && aligned16(dz_out);
+#define FX_SMCE(TT, TL, CAP_)                                                                                         \
+    softmax_ce_kernel<TT, TL, CAP_><<<(unsigned)rows, SM_THREADS, 0, stream>>>(                                        \
+        reinterpret_cast<const TT*>(logits), reinterpret_cast<TT*>(dz_out), reinterpret_cast<const TL*>(labels),      \
+        loss_mask, loss_out, max_idx_out, max_val_out, V, in_row_stride, out_row_stride, ignore_index, max_loss, vec, \
+        softcap)
     FX_DISPATCH_DTYPE(dt, TT,
-        if (labels_are_int64)
-            softmax_ce_kernel<TT, int64_t><<<(unsigned)rows, SM_THREADS, 0, stream>>>(reinterpret_cast<const TT*>(logits), reinterpret_cast<TT*>(dz_out), reinterpret_cast<const int64_t*>(labels), loss_mask, loss_out, max_idx_out, max_val_out, V, in_row_stride, out_row_stride, ignore_index, max_loss, vec);
-        else
-            softmax_ce_kernel<TT, int32_t><<<(unsigned)rows, SM_THREADS, 0, stream>>>(reinterpret_cast<const TT*>(logits), reinterpret_cast<TT*>(dz_out), reinterpret_cast<const int32_t*>(labels), loss_mask, loss_out, max_idx_out, max_val_out, V, in_row_stride, out_row_stride, ignore_index, max_loss, vec));
+        if (labels_are_int64) { if (softcap > 0.f) FX_SMCE(TT, int64_t, true); else FX_SMCE(TT, int64_t, false); }
+        else { if (softcap > 0.f) FX_SMCE(TT, int32_t, true); else FX_SMCE(TT, int32_t, false); });
+#undef FX_SMCE
     FX_CHECK_LAUNCH("fx_softmax_ce");
+    return 0;
+}
+
+static unsigned flat_grid(int64_t items) {
+    const int64_t g = (items + 255) / 256;
+    return (unsigned)(g < 1 ? 1 : (g > 65536 ? 65536 : g));
+}
+
+extern "C" int fx_softcap_fwd(void* logits, void* gate_out, int64_t rows, int V, int64_t row_stride,
+                              int64_t gate_row_stride, float softcap, int dt, hipStream_t stream) {
+    if (rows < 0 || V <= 0) FX_FAIL("fx_softcap_fwd: bad shape");
+    if (!(softcap > 0.f)) FX_FAIL("fx_softcap_fwd: softcap must be positive");
+    if (rows == 0) return 0;
+    if (!logits || !gate_out) FX_FAIL("fx_softcap_fwd: null pointer");
+    const bool vec = (V % 8 == 0) && (row_stride % 8 == 0) && (gate_row_stride % 8 == 0) && aligned16(logits) && aligned16(gate_out);
+    FX_DISPATCH_DTYPE(dt, TT,
+        softcap_fwd_kernel<TT><<<flat_grid(rows * (vec ? V / 8 : V)), 256, 0, stream>>>(
+            reinterpret_cast<TT*>(logits), reinterpret_cast<TT*>(gate_out), rows, V, row_stride, gate_row_stride, softcap, vec));
+    FX_CHECK_LAUNCH("fx_softcap_fwd");
+    return 0;
+}
+
+extern "C" int fx_softcap_bwd(void* dz, const void* gate, int64_t rows, int V, int64_t row_stride,
+                              int64_t gate_row_stride, int dt, hipStream_t stream) {
+    if (rows < 0 || V <= 0) FX_FAIL("fx_softcap_bwd: bad shape");
+    if (rows == 0) return 0;
+    if (!dz || !gate) FX_FAIL("fx_softcap_bwd: null pointer");
+    const bool vec = (V % 8 == 0) && (row_stride % 8 == 0) && (gate_row_stride % 8 == 0) && aligned16(dz) && aligned16(gate);
+    FX_DISPATCH_DTYPE(dt, TT,
+        softcap_bwd_kernel<TT><<<flat_grid(rows * (vec ? V / 8 : V)), 256, 0, stream>>>(
+            reinterpret_cast<TT*>(dz), reinterpret_cast<const TT*>(gate), rows, V, row_stride, gate_row_stride, vec));
+    FX_CHECK_LAUNCH("fx_softcap_bwd");
     return 0;
 }

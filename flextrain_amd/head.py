@@ -18,6 +18,7 @@ import torch
 from .loss import CrossEntropyLoss, LossFn, TokenContext
 from .matmul_dispatcher import CublasLtDispatcher
 from .ops.rmsnorm import flextrain_rmsnorm_bwd, flextrain_rmsnorm_fwd
+from .ops.softmax_ce import flextrain_logit_softcap_bwd, flextrain_logit_softcap_fwd
 
 
 @dataclass(frozen=True)
@@ -108,18 +109,22 @@ class LMHead:
             logits = logits_buf[:t_prime]
             disp.matmul(stream, A=head_in, B=w_head_proj, D=logits)
 
+            # Gemma's final-logit soft cap (flextrain/nn/head.py:273-298): a loss object that caps inside
+            # its own kernel gets the cap as an argument; for any other one the logits are capped in
+            # place first and dZ is multiplied by the saved gate afterwards, as the reference does.
             cap = cfg.final_logit_softcap
-            softcap_gate = None
-            if cap is not None and cap > 0.0:
-                inv_cap = 1.0 / float(cap)
-                logits.mul_(inv_cap).tanh_().mul_(float(cap))
-                ratio = logits * inv_cap
-                softcap_gate = (1.0 - ratio * ratio).to(logits.dtype)
-
-            dZ, aux = loss_fn.compute(logits, token_ctx.slice_for(offset, t_prime), loss_scale=loss_scale,
-                                      per_token_loss_out=per_token_loss[offset:offset + t_prime])
-            if softcap_gate is not None:
-                dZ.mul_(softcap_gate)
+            capped = cap is not None and cap > 0.0
+            token_slice = token_ctx.slice_for(offset, t_prime)
+            loss_out = per_token_loss[offset:offset + t_prime]
+            if capped and getattr(loss_fn, "supports_logit_softcap", False):
+                dZ, aux = loss_fn.compute(logits, token_slice, loss_scale=loss_scale, per_token_loss_out=loss_out,
+                                          logit_softcap=float(cap))
+            else:
+                gate = flextrain_logit_softcap_fwd(logits, float(cap)) if capped else None
+                dZ, aux = loss_fn.compute(logits, token_slice, loss_scale=loss_scale, per_token_loss_out=loss_out)
+                if gate is not None:
+                    flextrain_logit_softcap_bwd(dZ, gate)
+                    del gate
             if "next_prediction" in aux:
                 next_prediction[offset:offset + t_prime].copy_(aux.pop("next_prediction"))
                 next_prediction_prob[offset:offset + t_prime].copy_(aux.pop("next_prediction_prob"))

@@ -77,7 +77,13 @@ class CrossEntropyLoss:
         self.ignore_index = ignore_index
         self.fused = fused
 
-    def compute(self, logits, token_slice, *, loss_scale, per_token_loss_out):
+    @property
+    def supports_logit_softcap(self) -> bool:
+        """Whether ``compute`` takes ``logit_softcap=`` and applies the final-logit soft cap itself
+        (the fused kernel does, inside its two sweeps; the head then skips its own capping passes)."""
+        return self.fused
+
+    def compute(self, logits, token_slice, *, loss_scale, per_token_loss_out, logit_softcap=None):
         if token_slice.labels is None:
             raise ValueError("CrossEntropyLoss requires token_slice.labels")
         labels = token_slice.labels
@@ -87,8 +93,10 @@ class CrossEntropyLoss:
         if self.fused:
             dZ, _ = flextrain_softmax_cross_entropy(
                 logits, labels, L=per_token_loss_out, loss_mask=token_slice.loss_mask, max_idx_out=next_pred,
-                max_val_out=next_prob, ignore_index=self.ignore_index)
+                max_val_out=next_prob, ignore_index=self.ignore_index, logit_softcap=logit_softcap)
             return dZ, {"next_prediction": next_pred, "next_prediction_prob": next_prob}
+        if logit_softcap is not None:
+            raise ValueError("the unfused sequence does not cap logits; cap them before calling compute")
         ignore_rows = labels == self.ignore_index
         any_ignore = bool(ignore_rows.any().item())
         safe = torch.where(ignore_rows, torch.zeros_like(labels), labels) if any_ignore else labels

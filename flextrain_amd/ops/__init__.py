@@ -31,6 +31,8 @@ from .rmsnorm import (
 )
 from .softmax_ce import (
     flextrain_cross_entropy_loss,
+    flextrain_logit_softcap_bwd,
+    flextrain_logit_softcap_fwd,
     flextrain_softmax,
     flextrain_softmax_cross_entropy,
     flextrain_softmax_cross_entropy_loss,
@@ -91,6 +93,8 @@ __all__ = [
     "flextrain_rope_fwd",
     "flextrain_rope_partial_bwd",
     "flextrain_rope_partial_fwd",
+    "flextrain_logit_softcap_bwd",
+    "flextrain_logit_softcap_fwd",
     "flextrain_softmax",
     "flextrain_softmax_cross_entropy",
     "flextrain_softmax_cross_entropy_loss",

@@ -123,11 +123,15 @@ def flextrain_softmax_cross_entropy_loss(X, labels, L=None, Valid_Count=None):
 
 
 def flextrain_softmax_cross_entropy(logits, labels, L=None, dZ=None, loss_mask=None, max_idx_out=None,
-                                    max_val_out=None, ignore_index=-100, max_loss=100.0):
+                                    max_val_out=None, ignore_index=-100, max_loss=100.0, logit_softcap=None):
     """Fused row softmax + cross-entropy + dZ.  ``dZ`` defaults to ``logits`` (in
     place).  Per-row fp32 loss ``lse - logit[label]`` goes to ``L``; rows whose
     label is ``ignore_index`` or whose ``loss_mask`` is False get loss 0 and a zero
-    dZ row.  No host synchronisation.  Returns ``(dZ, L)``."""
+    dZ row.  No host synchronisation.  Returns ``(dZ, L)``.
+
+    ``logit_softcap`` (Gemma's final-logit soft cap, flextrain/nn/head.py:273-298): loss,
+    argmax and probabilities are taken from ``cap * tanh(logits / cap)`` and ``dZ`` is the
+    gradient at the uncapped logits; the capped logits are never written."""
     if logits.dim() != 2 or not logits.is_cuda:
         raise ValueError("logits must be a 2-D CUDA tensor")
     T, V = logits.shape
@@ -153,10 +157,51 @@ def flextrain_softmax_cross_entropy(logits, labels, L=None, dZ=None, loss_mask=N
     for t, nm, dt in ((max_idx_out, "max_idx_out", torch.int64), (max_val_out, "max_val_out", torch.float32)):
         if t is not None and (tuple(t.shape) != (T,) or t.dtype != dt or not t.is_contiguous()):
             raise ValueError(f"{nm} must be a contiguous {dt} tensor of shape ({T},)")
+    cap = 0.0
+    if logit_softcap is not None:
+        cap = float(logit_softcap)
+        if not cap > 0.0:
+            raise ValueError(f"logit_softcap must be positive, got {logit_softcap}")
     labels = labels.contiguous()
     rc = lib().fx_softmax_ce(ptr(logits), ptr(dZ), ptr(labels), _labels_flag(labels), ptr(mask), ptr(L),
                              ptr(max_idx_out), ptr(max_val_out), T, V, logits.stride(0), dZ.stride(0),
-                             int(ignore_index), float(max_loss), dtype_enum(logits.dtype),
+                             int(ignore_index), float(max_loss), cap, dtype_enum(logits.dtype),
                              stream_ptr(logits.device))
     check(rc, "fx_softmax_ce")
     return dZ, L
+
+
+def _softcap_args(t, name):
+    if t.dim() != 2 or not t.is_cuda or t.stride(1) != 1:
+        raise ValueError(f"{name} must be a 2-D CUDA tensor with unit column stride")
+    if t.dtype not in _FLOATS:
+        raise TypeError(f"{name} dtype {t.dtype} not supported. Supported: {_FLOATS}")
+
+
+def flextrain_logit_softcap_fwd(logits, cap, gate_out=None):
+    """In place ``logits = cap * tanh(logits / cap)``; returns the gate
+    ``1 - (logits_capped / cap)^2`` in the logits' dtype (flextrain/nn/head.py:276-282)."""
+    _softcap_args(logits, "logits")
+    if not float(cap) > 0.0:
+        raise ValueError(f"cap must be positive, got {cap}")
+    if gate_out is None:
+        gate_out = torch.empty_like(logits)
+    elif gate_out.shape != logits.shape or gate_out.dtype != logits.dtype or gate_out.stride(1) != 1:
+        raise ValueError("gate_out must match logits in shape and dtype with unit column stride")
+    T, V = logits.shape
+    rc = lib().fx_softcap_fwd(ptr(logits), ptr(gate_out), T, V, logits.stride(0), gate_out.stride(0), float(cap),
+                              dtype_enum(logits.dtype), stream_ptr(logits.device))
+    check(rc, "fx_softcap_fwd")
+    return gate_out
+
+
+def flextrain_logit_softcap_bwd(dZ, gate):
+    """In place ``dZ *= gate`` (flextrain/nn/head.py:295-297)."""
+    _softcap_args(dZ, "dZ")
+    if gate.shape != dZ.shape or gate.dtype != dZ.dtype or gate.stride(1) != 1 or not gate.is_cuda:
+        raise ValueError("gate must match dZ in shape and dtype with unit column stride")
+    T, V = dZ.shape
+    rc = lib().fx_softcap_bwd(ptr(dZ), ptr(gate), T, V, dZ.stride(0), gate.stride(0), dtype_enum(dZ.dtype),
+                              stream_ptr(dZ.device))
+    check(rc, "fx_softcap_bwd")
+    return dZ

@@ -241,11 +241,23 @@ int fx_cross_entropy(void* probs, const void* labels, int labels_are_int64, floa
  * dZ out (dz_out may alias logits), per-row fp32 loss from the log-sum-exp
  * (lse - logit[label], clamped to max_loss), rows with label == ignore_index or a
  * zero loss_mask byte get loss 0 and a zero dZ row.  loss_mask (one byte per row),
- * max_idx_out and max_val_out are optional. */
+ * max_idx_out and max_val_out are optional.
+ * softcap > 0 folds the final-logit soft cap of flextrain/nn/head.py:273-298 into both
+ * sweeps: statistics, loss, argmax and probabilities are those of
+ * y = softcap * tanh(logit / softcap) (rounded to the storage type), and dZ is the gradient
+ * at the uncapped logit, (softmax(y) - onehot) * (1 - (y / softcap)^2).  0 = no cap. */
 int fx_softmax_ce(const void* logits, void* dz_out, const void* labels, int labels_are_int64,
                   const uint8_t* loss_mask, float* loss_out, int64_t* max_idx_out, float* max_val_out, int64_t rows,
-                  int V, int64_t in_row_stride, int64_t out_row_stride, int64_t ignore_index, float max_loss, int dt,
-                  hipStream_t stream);
+                  int V, int64_t in_row_stride, int64_t out_row_stride, int64_t ignore_index, float max_loss,
+                  float softcap, int dt, hipStream_t stream);
+
+/* The soft cap as passes of its own, for loss objects other than the fused kernel
+ * (flextrain/nn/head.py:276-282 and :295-297): fx_softcap_fwd caps logits in place and writes
+ * gate = 1 - (y / softcap)^2 in the storage type; fx_softcap_bwd multiplies dz by gate. */
+int fx_softcap_fwd(void* logits, void* gate_out, int64_t rows, int V, int64_t row_stride, int64_t gate_row_stride,
+                   float softcap, int dt, hipStream_t stream);
+int fx_softcap_bwd(void* dz, const void* gate, int64_t rows, int V, int64_t row_stride, int64_t gate_row_stride,
+                   int dt, hipStream_t stream);
 
 /* ---- Expert-grouped GEMMs -------------------------------------------------- */
 

@@ -14,7 +14,9 @@ only through the GEMM alpha (head.py:325-346).
 rounding of the probabilities to the output dtype.
 
 Pinned by tests/test_oracle_linear_ce.py: torch.softmax / argmax,
-F.cross_entropy(reduction="none"/"sum") and torch.autograd through the whole head.
+F.cross_entropy(reduction="none"/"sum") and torch.autograd through the whole head,
+with and without the final-logit soft cap (autograd through
+``F.cross_entropy(cap * tanh(logits / cap))``).
 """
 from __future__ import annotations
 
@@ -49,9 +51,22 @@ def cross_entropy_from_probs(p, labels, max_loss=100.0):
     return dz, loss, valid.float()
 
 
-def softmax_ce(logits, labels, loss_mask=None, ignore_index=-100, max_loss=100.0):
-    """The fused op: -> (dZ in logits.dtype, loss fp32, argmax, max prob)."""
+def softcap(logits, cap):
+    """Final-logit soft cap of flextrain/nn/head.py:273-282: -> (capped logits in logits.dtype,
+    gate = 1 - (capped / cap)^2 in fp32, from the ROUNDED capped logits as the reference computes it)."""
+    y = (torch.tanh(logits.float() / cap) * cap).to(logits.dtype)
+    r = y.float() / cap
+    return y, 1.0 - r * r
+
+
+def softmax_ce(logits, labels, loss_mask=None, ignore_index=-100, max_loss=100.0, logit_softcap=None):
+    """The fused op: -> (dZ in logits.dtype, loss fp32, argmax, max prob).  With ``logit_softcap`` the
+    loss, argmax and probabilities are those of the capped logits and dZ is chained through the cap's
+    derivative (flextrain/nn/head.py:295-297), i.e. the gradient at the uncapped logits."""
     T, V = logits.shape
+    gate = None
+    if logit_softcap is not None:
+        logits, gate = softcap(logits, logit_softcap)
     z = logits.float()
     lab = labels.long()
     keep = lab != ignore_index
@@ -65,12 +80,14 @@ def softmax_ce(logits, labels, loss_mask=None, ignore_index=-100, max_loss=100.0
     hot = keep & valid
     dz[torch.arange(T)[hot], safe[hot]] -= 1.0
     dz = dz * keep[:, None].float()
+    if gate is not None:
+        dz = dz * gate
     _, first, mx = softmax(logits)
     return dz.to(logits.dtype), loss, first, mx
 
 
 def head_forward_backward(x, w_norm, w_head, labels, eps=1e-5, chunk=1024, loss_scale=1.0, loss_mask=None,
-                          g_head=None, g_norm=None, ignore_index=-100):
+                          g_head=None, g_norm=None, ignore_index=-100, logit_softcap=None):
     """x (T,d) compute dtype; w_head (d,V); returns dict(dx, per_token_loss, g_head fp32, g_norm fp32,
     next_prediction, next_prediction_prob)."""
     T, d = x.shape
@@ -88,7 +105,7 @@ def head_forward_backward(x, w_norm, w_head, labels, eps=1e-5, chunk=1024, loss_
         h, rstd = o_norm.rmsnorm_fwd(x[s], w_norm, eps)
         logits = (h.float() @ wf).to(dt)
         dz, loss[s], pred[s], prob[s] = softmax_ce(logits, labels[s], None if loss_mask is None else loss_mask[s],
-                                                   ignore_index)
+                                                   ignore_index, logit_softcap=logit_softcap)
         gh += loss_scale * (h.float().t() @ dz.float())
         dh = (loss_scale * (dz.float() @ wf.t())).to(dt)
         dx[s], gn, _ = o_norm.rmsnorm_bwd(dh, x[s], w_norm, rstd, dw_old=gn)

@@ -77,3 +77,56 @@ def test_head_matches_autograd_and_is_chunk_independent():
     r2 = o_ce.head_forward_backward(x, w_norm, w_head, labels, loss_scale=2.0, g_head=r1["g_head"])
     torch.testing.assert_close(r2["dx"], 2 * r1["dx"], rtol=1e-5, atol=1e-7)
     torch.testing.assert_close(r2["g_head"], 3 * r1["g_head"], rtol=1e-5, atol=1e-6)
+
+
+def test_softcap_oracle_matches_autograd_through_capped_cross_entropy():
+    """fp32 inputs (no rounding of the capped logits): the oracle's loss and dZ against autograd
+    through F.cross_entropy(cap * tanh(logits / cap)); a dropped gate, a gate taken from the uncapped
+    logits or a cap applied after the softmax all fail here."""
+    g = gen(31)
+    cap = 30.0
+    x = randn(g, 40, 257, dtype=torch.float32, std=25.0).requires_grad_()      # well into the saturating range
+    labels = torch.randint(0, 257, (40,), generator=g)
+    labels[::7] = -100
+    mask = torch.ones(40, dtype=torch.bool)
+    mask[2] = False
+    capped = torch.tanh(x / cap) * cap
+    per_token = F.cross_entropy(capped, labels, ignore_index=-100, reduction="none") * mask
+    (gx,) = torch.autograd.grad(per_token.sum(), x)
+    dz, loss, idx, mx = o_ce.softmax_ce(x.detach(), labels, mask, logit_softcap=cap)
+    torch.testing.assert_close(loss, per_token.detach(), rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(dz, gx, rtol=1e-4, atol=1e-7)
+    assert torch.equal(idx, capped.detach().argmax(-1))
+    torch.testing.assert_close(mx, torch.softmax(capped.detach(), -1).max(-1).values, rtol=1e-5, atol=0)
+    # the two-pass form of the reference (cap in place, loss, multiply by the saved gate) is the same thing
+    y, gate = o_ce.softcap(x.detach(), cap)
+    dz2, loss2, _, _ = o_ce.softmax_ce(y, labels, mask)
+    torch.testing.assert_close(dz2 * gate, dz, rtol=1e-6, atol=1e-9)
+    torch.testing.assert_close(loss2, loss, rtol=0, atol=0)
+    # a very large cap is no cap
+    dz3, loss3, _, _ = o_ce.softmax_ce(x.detach() * 0.01, labels, mask, logit_softcap=1e6)
+    dz4, loss4, _, _ = o_ce.softmax_ce(x.detach() * 0.01, labels, mask)
+    torch.testing.assert_close(dz3, dz4, rtol=1e-4, atol=1e-7)
+    torch.testing.assert_close(loss3, loss4, rtol=1e-4, atol=1e-5)
+
+
+def test_head_with_softcap_matches_autograd():
+    g = gen(32)
+    T, d, V, cap = 40, 32, 150, 5.0
+    x = randn(g, T, d, dtype=torch.float32)
+    w_norm = randn(g, d, dtype=torch.float32, std=0.1, mean=1.0)
+    w_head = randn(g, d, V, dtype=torch.float32, std=1.0)               # logits of a few units: the cap bites
+    labels = torch.randint(0, V, (T,), generator=g)
+    labels[torch.rand(T, generator=g) < 0.1] = -100
+    scale = 1.0 / int((labels != -100).sum())
+    xa, wn, wh = x.clone().requires_grad_(), w_norm.clone().requires_grad_(), w_head.clone().requires_grad_()
+    logits = F.rms_norm(xa, (d,), wn, eps=1e-5) @ wh
+    assert float(logits.detach().abs().max()) > cap
+    loss = F.cross_entropy(torch.tanh(logits / cap) * cap, labels, ignore_index=-100, reduction="sum") * scale
+    gx, gn, gh = torch.autograd.grad(loss, (xa, wn, wh))
+    for chunk in (40, 16):
+        r = o_ce.head_forward_backward(x, w_norm, w_head, labels, chunk=chunk, loss_scale=scale, logit_softcap=cap)
+        torch.testing.assert_close(r["per_token_loss"].sum() * scale, loss.detach(), rtol=1e-5, atol=1e-6)
+        torch.testing.assert_close(r["dx"], gx, rtol=1e-4, atol=1e-6)
+        torch.testing.assert_close(r["g_head"], gh, rtol=1e-4, atol=1e-6)
+        torch.testing.assert_close(r["g_norm"], gn, rtol=1e-4, atol=1e-6)
