@@ -396,21 +396,38 @@ def run_lm_head(torch, dev, stream, rn):
     labels[torch.rand(T, device=dev) < 0.1] = -100
     g_store = torch.zeros(V, d, dtype=torch.float32, device=dev)
     g_norm = torch.zeros(d, dtype=torch.float32, device=dev)
-    head = LMHead(LMHeadConfig(d_model=d, vocab_size=V, head_chunk_size=chunk))
+    head = None
+    grads = {"g_head_proj": g_store.t(), "g_final_norm": g_norm}
     scale = 1.0 / int((labels != -100).sum())
     x = x0.clone()
 
     def run():
         x.copy_(x0)
         head.forward_backward(x, TokenContext(labels=labels), None, {"w_final_norm": w_norm, "w_head_proj": w.t()},
-                              {"g_head_proj": g_store.t(), "g_final_norm": g_norm}, None, loss_scale=scale)
+                              grads, None, loss_scale=scale)
 
     rows = []
-    ms = _time_launches(torch, stream, [run], warmup=1, reps=3)
-    rows.append(_op_entry("c3.lm_head fwd+bwd (chunk 1024 x 8 fused per GEMM group, fp32 dW)", 6 * T * d * V, "TFLOP/s", ms))
-    head = LMHead(LMHeadConfig(d_model=d, vocab_size=V, head_chunk_size=chunk, fuse_chunks=1))
-    ms = _time_launches(torch, stream, [run], warmup=1, reps=3)
-    rows.append(_op_entry("c3.lm_head fwd+bwd (chunk 1024, one GEMM group per chunk as the reference, fp32 dW)", 6 * T * d * V, "TFLOP/s", ms))
+    chunk_bytes = chunk * V * 2
+    g_bf16 = torch.zeros(V, d, dtype=torch.bfloat16, device=dev)
+
+    def head_row(name, fuse, g_head):
+        nonlocal head
+        head = LMHead(LMHeadConfig(d_model=d, vocab_size=V, head_chunk_size=chunk, fuse_chunks=fuse))
+        grads["g_head_proj"] = g_head.t()
+        ms = _time_launches(torch, stream, [run], warmup=1, reps=3)
+        row = _op_entry(name, 6 * T * d * V, "TFLOP/s", ms)
+        groups = fuse if fuse is not None else max(1, head.cfg.logits_buffer_bytes // chunk_bytes)
+        row["logits_buffer_MB"] = round(groups * chunk_bytes / 1e6)
+        row["head_gradient"] = str(g_head.dtype).replace("torch.", "")
+        rows.append(row)
+
+    # The reference's own schedule and gradient type first (one 1024-token logits buffer; torch.addmm
+    # into a compute-dtype accumulator, flextrain/nn/head.py:82-84, :324-331), then the same with the
+    # fp32 accumulator this package also takes, then larger GEMM groups.
+    head_row("c3.lm_head fwd+bwd (chunk 1024, one GEMM group per chunk and bf16 dW += as the reference)", 1, g_bf16)
+    head_row("c3.lm_head fwd+bwd (chunk 1024, one GEMM group per chunk, fp32 dW +=)", 1, g_store)
+    head_row("c3.lm_head fwd+bwd (chunk 1024 x 2 per GEMM group: the default, fp32 dW +=)", None, g_store)
+    head_row("c3.lm_head fwd+bwd (chunk 1024 x 8 per GEMM group, fp32 dW +=)", 8, g_store)
     # the three GEMMs of one micro-chunk, timed alone
     disp = CublasLtDispatcher()
     sp = stream.cuda_stream
@@ -424,6 +441,9 @@ def run_lm_head(torch, dev, stream, rn):
     ms = _time_launches(torch, stream, [lambda: disp.matmul_fast(sp, logits.t(), h, C=gt, D=gt, alpha=scale, beta=1.0)],
                         warmup=2, reps=10)
     rows.append(_op_entry("c3.dW gemm [128256,1024]x[1024,4096] (+= fp32)", 2 * chunk * d * V, "TFLOP/s", ms))
+    ms = _time_launches(torch, stream, [lambda: disp.matmul_fast(sp, logits.t(), h, C=g_bf16, D=g_bf16, alpha=scale, beta=1.0)],
+                        warmup=2, reps=10)
+    rows.append(_op_entry("c3.dW gemm [128256,1024]x[1024,4096] (+= bf16)", 2 * chunk * d * V, "TFLOP/s", ms))
     ms = _time_launches(torch, stream, [lambda: disp.matmul_fast(sp, logits, w, D=dxh)], warmup=2, reps=10)
     rows.append(_op_entry("c3.dX gemm [1024,128256]x[128256,4096]", 2 * chunk * d * V, "TFLOP/s", ms))
     # For comparison only (not a product path): the vendor BLAS, which the reference's cuBLASLt
@@ -446,7 +466,7 @@ def run_lm_head(torch, dev, stream, rn):
     row["achieved_by_minimal_bytes"] = minimal["achieved"]
     row["frac_by_minimal_bytes"] = minimal["frac"]
     rows.append(row)
-    del w, g_store, logits, x, x0
+    del w, g_store, g_bf16, logits, x, x0
     torch.cuda.empty_cache()
     return rows
 

@@ -48,6 +48,7 @@ struct OperandView {
     // Gathered rows (K-contiguous A tiles of the loaders that say so): tile row r is row
     // row_map[origin + r] of `base` instead of row origin + r.
     const int32_t* row_map = nullptr;
+    int map_rows = 0;          // rows of `base` a gathered tile may address: map entries are clamped to [0, map_rows)
     // tile row -> which matrix, and the index offset from `origin`
     __device__ __forceinline__ bool dual_second(int r) const { return (r & half) != 0; }
     __device__ __forceinline__ int dual_index(int r) const { return ((r & ~(2 * half - 1)) >> 1) + (r & (half - 1)); }

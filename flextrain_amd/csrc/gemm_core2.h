@@ -311,7 +311,9 @@ struct TileLoader {
                 g = g < op.ext ? g : op.ext - 1;
                 // gathered: the offset is taken from the start of the source matrix (the caller checks
                 // that the whole source stays below 4 GB)
-                const int64_t row = gathered ? (int64_t)op.row_map[g] : (int64_t)(g - op.origin);
+                // a map entry outside the source (a mapping that is no permutation, an unwritten entry)
+                // must not turn into an address outside it
+                const int64_t row = gathered ? (int64_t)min(max(op.row_map[g], 0), op.map_rows - 1) : (int64_t)(g - op.origin);
                 off[j] = (unsigned)((row * op.ld + (pos ^ swz(r)) * 8) * (int64_t)sizeof(T));
             }
             base = gathered ? op.base : op.base + (int64_t)op.origin * op.ld;
@@ -394,7 +396,7 @@ constexpr size_t epilogue_lds_bytes() { return (size_t)NW * 32 * (WN + 4) * size
 // loads issued so far are waited for just before the last band's stores go out (a wait placed after
 // the epilogue would also wait for every store to drain, because loads and stores share one counter:
 // here the earlier bands' stores have had most of the epilogue to complete).
-template <typename T, typename TD, int WM, int WN, bool LOADS_LAND = false>
+template <typename T, typename TD, int WM, int WN, bool LOADS_LAND = false, bool NT = false>
 FX_DEV void epilogue_tile(f32x16_t (&acc)[WM / 32][WN / 32], const TD* C, TD* D, int64_t ldc, int64_t ldd, int row_base,
                           int col_base, int M, int N, float alpha, float beta, T* smem, int wave, int lane) {
     constexpr int TM = WM / 32, TN = WN / 32;
@@ -425,8 +427,10 @@ FX_DEV void epilogue_tile(f32x16_t (&acc)[WM / 32][WN / 32], const TD* C, TD* D,
                     const int row = row_base + (i + b) * 32 + id / GROUPS, col = col_base + (id % GROUPS) * 8;
                     if (row < M && col + 8 <= N) {
 #pragma unroll
-                        for (int q = 0; q < CVN; ++q)
-                            cpre[b][t][q] = *reinterpret_cast<const CV*>(C + (int64_t)row * ldc + col + q * VecOf<TD>::N);
+                        for (int q = 0; q < CVN; ++q) {
+                            const CV* src = reinterpret_cast<const CV*>(C + (int64_t)row * ldc + col + q * VecOf<TD>::N);
+                            cpre[b][t][q] = NT ? __builtin_nontemporal_load(src) : *src;
+                        }
                     }
                 }
         }
@@ -459,7 +463,7 @@ FX_DEV void epilogue_tile(f32x16_t (&acc)[WM / 32][WN / 32], const TD* C, TD* D,
                         for (int e = 0; e < VecOf<TD>::N; ++e)
                             o[q * VecOf<TD>::N + e] += beta * (float)cpre[i % CB][t][q][e];
                 }
-                store_f32<TD, 8>(dst, o);
+                store_f32<TD, 8, NT>(dst, o);
             } else {
                 for (int e = 0; e < 8 && col + e < N; ++e) {
                     float r = o[e];
@@ -624,7 +628,7 @@ FX_DEV void gemm_mainloop2(const OperandView<T>& A, const OperandView<T>& B, int
     static_assert(gemm2_lds_bytes<T, BM, BN, WAVES_M, WAVES_N>() <= 160 * 1024, "tile configuration exceeds the 160 KB of LDS");
 }
 
-template <typename T, typename TD, int BM, int BN, int WAVES_M, int WAVES_N, bool A_MN, bool B_MN>
+template <typename T, typename TD, int BM, int BN, int WAVES_M, int WAVES_N, bool A_MN, bool B_MN, bool NT = false>
 FX_DEV void gemm_tile2(const OperandView<T>& A, const OperandView<T>& B, const TD* C, TD* D, int64_t ldc,
                        int64_t ldd, int M, int N, int K, float alpha, float beta, T* smem) {
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
@@ -632,7 +636,7 @@ FX_DEV void gemm_tile2(const OperandView<T>& A, const OperandView<T>& B, const T
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
     f32x16_t acc[WM / 32][WN / 32];
     gemm_mainloop2<T, BM, BN, WAVES_M, WAVES_N, A_MN, B_MN>(A, B, K, smem, acc);
-    epilogue_tile<T, TD, WM, WN>(acc, C, D, ldc, ldd, A.origin + wm * WM, B.origin + wn * WN, M, N, alpha, beta, smem, wave, lane);
+    epilogue_tile<T, TD, WM, WN, false, NT>(acc, C, D, ldc, ldd, A.origin + wm * WM, B.origin + wn * WN, M, N, alpha, beta, smem, wave, lane);
 }
 
 // Two GEMMs that share A, fused with the gated activation:
@@ -640,7 +644,7 @@ FX_DEV void gemm_tile2(const OperandView<T>& A, const OperandView<T>& B, const T
 // with (gate, value) = (P1, P2) when gate_first, else (P2, P1), evaluated from the ROUNDED P1 / P2
 // exactly as a separate activation kernel reading them back would.  The workgroup covers BN/2
 // columns of each product.  Needs K % 64 == 0, Nh % 8 == 0, 16-byte aligned rows.
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_MN, bool B_MN, bool B_DUAL = false>
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_MN, bool B_MN, bool B_DUAL = false, bool ZERO = true>
 FX_DEV void gemm_mainloop32(const OperandView<T>& A, const OperandView<T>& B, int K, T* smem,
                             f32x16_t (&acc)[BM / WAVES_M / 32][BN / WAVES_N / 32]);
 
@@ -787,7 +791,7 @@ struct Tile32Loader {
                 const int r = (j * NW + wave) * 16 + rr;
                 int g = op.origin + (DUAL ? op.dual_index(r) : r);
                 g = g < op.ext ? g : op.ext - 1;
-                const int64_t row = gathered ? (int64_t)op.row_map[g] : (int64_t)(g - op.origin);
+                const int64_t row = gathered ? (int64_t)min(max(op.row_map[g], 0), op.map_rows - 1) : (int64_t)(g - op.origin);
                 off[j] = (unsigned)((row * op.ld + (pos ^ swz_k<32>(r)) * 8) * (int64_t)sizeof(T));
             }
             base = gathered ? op.base : op.base + (int64_t)op.origin * op.ld;
@@ -829,7 +833,8 @@ constexpr size_t gemm32_lds_bytes() {
 
 // K loop with 32-wide steps over three rotating LDS stages; K must be a multiple of 32.
 // Leaves the accumulators in `acc` and ends with a barrier (the stages become epilogue staging).
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_MN, bool B_MN, bool B_DUAL>
+// ZERO = false: `acc` already holds partial sums and is added to.
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_MN, bool B_MN, bool B_DUAL, bool ZERO>
 FX_DEV void gemm_mainloop32(const OperandView<T>& A, const OperandView<T>& B, int K, T* smem,
                             f32x16_t (&acc)[BM / WAVES_M / 32][BN / WAVES_N / 32]) {
     constexpr int NW = WAVES_M * WAVES_N;
@@ -840,12 +845,14 @@ FX_DEV void gemm_mainloop32(const OperandView<T>& A, const OperandView<T>& B, in
     static_assert((BM + BN) * 64 % (1024 * NW) == 0, "loads must split evenly over the waves");
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    if (ZERO) {
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
+            for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+    }
     const int n = K / 32;
     constexpr bool B_FN = B_MN && B_DUAL;                 // the one tile form without a scalar-base loader
     typedef Tile32Loader<T, BM, NW, A_MN, false> LoadA;

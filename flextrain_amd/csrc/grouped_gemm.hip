@@ -16,8 +16,12 @@
 
 namespace fx {
 
-// Workspace layout (int32): [0] number of tiles, [1 .. E+1] row offsets (E+1 entries),
-// then (expert, first_row_in_expert) pairs, one per BM-row tile.
+// Workspace layout (int32): [0] number of tiles, [1] E and [2] tile height BM the plan was made
+// for, [3 .. E+3] row offsets (E+1 entries), then (expert, first_row_in_expert) pairs, one per
+// BM-row tile.  A launch that is given no counts takes the plan as it finds it: the kernels compare
+// [1] and [2] with their own E and tile height and do nothing when they differ (a workspace that
+// was never planned, or was planned for another shape, must not send them out of bounds), and
+// never walk more tiles than the host computed as the worst case.
 struct GroupedWs {
     int32_t* ntiles;
     int32_t* offsets;
@@ -26,7 +30,15 @@ struct GroupedWs {
 
 static inline GroupedWs split_ws(void* ws, int E) {
     int32_t* p = reinterpret_cast<int32_t*>(ws);
-    return GroupedWs{p, p + 1, p + 2 + E};
+    return GroupedWs{p, p + 3, p + 4 + E};
+}
+
+// Number of (row tile, column tile) pairs to process, 0 when the plan is not for (E, BM).
+FX_DEV int plan_total(const int32_t* NTILES, int E, int BM, int tiles_n, int max_tiles) {
+    if (NTILES[1] != E || (BM != 0 && NTILES[2] != BM)) return 0;
+    int nt = NTILES[0];
+    nt = nt < 0 ? 0 : (nt > max_tiles ? max_tiles : nt);
+    return nt * tiles_n;
 }
 
 __global__ __launch_bounds__(256) void grouped_plan_kernel(const int32_t* __restrict__ COUNTS, int E, int BM,
@@ -65,7 +77,7 @@ __global__ __launch_bounds__(256) void grouped_plan_kernel(const int32_t* __rest
         if (threadIdx.x == 255) { carry_r = br + ir; carry_t = bt + it; }
         __syncthreads();
     }
-    if (threadIdx.x == 0) { OFFSETS[E] = carry_r; NTILES[0] = carry_t; }
+    if (threadIdx.x == 0) { OFFSETS[E] = carry_r; NTILES[0] = carry_t; NTILES[1] = E; NTILES[2] = BM; }
 }
 
 template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool B_MN>
@@ -73,14 +85,14 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void grouped_rows_kernel(
     const T* __restrict__ A, int64_t lda, const T* __restrict__ B, int64_t ldb, int64_t b_expert_stride,
     const T* C, int64_t ldc, T* D, int64_t ldd, const int32_t* __restrict__ NTILES,
     const int32_t* __restrict__ OFFSETS, const int32_t* __restrict__ TILES, int N, int K, float alpha,
-    float beta, int tiles_n) {
+    float beta, int tiles_n, int E, int max_tiles) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T* smem = reinterpret_cast<T*>(smem_raw);
     // The grid is sized for the worst case; the live tiles are (row tile, column tile) pairs in
     // expert-major order with the column tile fastest.  Workgroups are dealt round-robin to the 8
     // XCDs: give each XCD a contiguous band of that order, so the workgroups that share an expert's
     // weights and a row tile's activations meet in one L2.
-    const int total = NTILES[0] * tiles_n;
+    const int total = plan_total(NTILES, E, BM, tiles_n, max_tiles);
     const int pid = blockIdx.x;
     if (pid >= total) return;
     const int p = xcd_band(pid, total);
@@ -102,10 +114,10 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64, 2) void grouped_rows_kernel
     const T* __restrict__ A, int64_t lda, const T* __restrict__ B, int64_t ldb, int64_t b_expert_stride,
     const T* C, int64_t ldc, T* D, int64_t ldd, const int32_t* __restrict__ NTILES,
     const int32_t* __restrict__ OFFSETS, const int32_t* __restrict__ TILES, int N, int K, float alpha,
-    float beta, int tiles_n) {
+    float beta, int tiles_n, int E, int max_tiles) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T* smem = reinterpret_cast<T*>(smem_raw);
-    const int total = NTILES[0] * tiles_n;
+    const int total = plan_total(NTILES, E, BM, tiles_n, max_tiles);
     const int pid = blockIdx.x;
     if (pid >= total) return;
     const int p = xcd_band(pid, total);
@@ -133,10 +145,10 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64, K32 ? 2 : 1) void grouped_r
     const T* __restrict__ A, int64_t lda, const T* __restrict__ B, int64_t ldb, int64_t b_expert_stride,
     int64_t b2_delta, T* P1, T* P2, int64_t ldp, T* ACTO, int64_t ldact, const int32_t* __restrict__ NTILES,
     const int32_t* __restrict__ OFFSETS, const int32_t* __restrict__ TILES, int Nh, int K, int gate_first,
-    int tiles_n, const int32_t* __restrict__ A_ROW_MAP) {
+    int tiles_n, const int32_t* __restrict__ A_ROW_MAP, int a_rows, int E, int max_tiles) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T* smem = reinterpret_cast<T*>(smem_raw);
-    const int total = NTILES[0] * tiles_n;
+    const int total = plan_total(NTILES, E, BM, tiles_n, max_tiles);
     const int pid = blockIdx.x;
     if (pid >= total) return;
     const int p = xcd_band(pid, total);
@@ -148,7 +160,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64, K32 ? 2 : 1) void grouped_r
     // A_ROW_MAP: expert-sorted row r is row A_ROW_MAP[r] of A (the token it was routed from): the
     // rows are gathered by the tile loads themselves and no expert-sorted copy of A exists
     OperandView<T> a{A_ROW_MAP ? A : A + row0 * lda, lda, rows, m0};
-    if (A_ROW_MAP) a.row_map = A_ROW_MAP + row0;
+    if (A_ROW_MAP) { a.row_map = A_ROW_MAP + row0; a.map_rows = a_rows; }
     const T* b1 = B + (int64_t)e * b_expert_stride;
     OperandView<T> b{b1, ldb, Nh, tn * (BN / 2), BN / WAVES_N / 2, b1 + b2_delta};
     gemm_tile2_glu<T, BM, BN, WAVES_M, WAVES_N, B_MN, ACT_SILU, K32>(a, b, P1 + row0 * ldp, P2 + row0 * ldp, ldp,
@@ -177,12 +189,12 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void grouped_rows_walk_kern
     const T* __restrict__ A, int64_t lda, const T* __restrict__ B, int64_t ldb, int64_t b_expert_stride,
     const T* C, int64_t ldc, T* D, int64_t ldd, const int32_t* __restrict__ NTILES,
     const int32_t* __restrict__ OFFSETS, const int32_t* __restrict__ TILES, int N, int K, float alpha,
-    float beta, int tiles_n) {
+    float beta, int tiles_n, int E, int max_tiles) {
     static_assert((BM + BN) * GEMM_BK * sizeof(T) == 64 * 1024, "the LDS plan assumes 64 KB stages");
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T* smem = reinterpret_cast<T*>(smem_raw);
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
-    const int total = NTILES[0] * tiles_n;
+    const int total = plan_total(NTILES, E, BM, tiles_n, max_tiles);
     int pid = blockIdx.x;
     if (pid >= total) return;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -230,14 +242,14 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void grouped_rows_walk_kern
 template <typename T, typename TG, int BM, int BN, int WAVES_M, int WAVES_N>
 __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void grouped_wgrad_walk_kernel(
     const T* __restrict__ A, int64_t lda, const T* __restrict__ B, int64_t ldb, TG* G, int64_t ldg,
-    int64_t g_expert_stride, const int32_t* __restrict__ OFFSETS, int M, int N, float alpha, float beta,
-    int tiles_n, int tiles_per_expert, int total) {
+    int64_t g_expert_stride, const int32_t* __restrict__ NTILES, const int32_t* __restrict__ OFFSETS, int M, int N,
+    float alpha, float beta, int tiles_n, int tiles_per_expert, int total, int E) {
     static_assert((BM + BN) * GEMM_BK * sizeof(T) == 64 * 1024, "the LDS plan assumes 64 KB stages");
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T* smem = reinterpret_cast<T*>(smem_raw);
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     int pid = blockIdx.x;
-    if (pid >= total) return;
+    if (pid >= total || NTILES[1] != E) return;      // only the row offsets of the plan are used: any tile height serves
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     struct Tile { int e, tm, tn, rows; int64_t row0; };
     auto lookup = [&](int id) {
@@ -307,7 +319,7 @@ static int walk_grid() {
 extern "C" size_t fx_grouped_ws_bytes(int E, int64_t total_rows) {
     if (E <= 0 || total_rows < 0) return 0;
     // smallest row tile is 128: at most total_rows/128 + E tiles
-    return sizeof(int32_t) * (size_t)(2 + E + 2 * (total_rows / 128 + E + 1));
+    return sizeof(int32_t) * (size_t)(4 + E + 2 * (total_rows / 128 + E + 1));
 }
 
 // Row tile: 256 x 256 (one workgroup per CU, 64-wide K-steps) when experts average 384 rows or
@@ -359,7 +371,7 @@ extern "C" int fx_grouped_gemm_rows(const void* A, int64_t lda, const void* B, i
         kern<<<dim3(max_tiles * (unsigned)tiles_n), WM_ * WN_ * 64, lds, stream>>>(                       \
             reinterpret_cast<const TT*>(A), lda, reinterpret_cast<const TT*>(B), ldb, b_expert_stride,    \
             reinterpret_cast<const TT*>(C), ldc, reinterpret_cast<TT*>(D), ldd, w.ntiles, w.offsets,      \
-            w.tiles, N, K, alpha, beta, tiles_n);                                                         \
+            w.tiles, N, K, alpha, beta, tiles_n, E, (int)max_tiles);                                      \
     }
 #define FX_ROWS32(TT, BMN)                                                                               \
     {                                                                                                     \
@@ -370,7 +382,7 @@ extern "C" int fx_grouped_gemm_rows(const void* A, int64_t lda, const void* B, i
         kern<<<dim3(max_tiles * (unsigned)tiles_n), 256, lds, stream>>>(                                  \
             reinterpret_cast<const TT*>(A), lda, reinterpret_cast<const TT*>(B), ldb, b_expert_stride,    \
             reinterpret_cast<const TT*>(C), ldc, reinterpret_cast<TT*>(D), ldd, w.ntiles, w.offsets,      \
-            w.tiles, N, K, alpha, beta, tiles_n);                                                         \
+            w.tiles, N, K, alpha, beta, tiles_n, E, (int)max_tiles);                                      \
     }
     if (BM == 128 && (K & 31) == 0) {   // small experts: 128 x 256 tiles, 32-wide K-steps, two workgroups per CU
         if (dt == DT_BF16) { if (trans_b) FX_ROWS32(bf16, false) else FX_ROWS32(bf16, true) }
@@ -388,7 +400,7 @@ extern "C" int fx_grouped_gemm_rows(const void* A, int64_t lda, const void* B, i
         kern<<<dim3(grid), 512, kWalkLdsBytes, stream>>>(                                                 \
             reinterpret_cast<const TT*>(A), lda, reinterpret_cast<const TT*>(B), ldb, b_expert_stride,    \
             reinterpret_cast<const TT*>(C), ldc, reinterpret_cast<TT*>(D), ldd, w.ntiles, w.offsets,      \
-            w.tiles, N, K, alpha, beta, tiles_n);                                                         \
+            w.tiles, N, K, alpha, beta, tiles_n, E, (int)max_tiles);                                      \
     }
 #define FX_ROWS_T(TT)                                                                                     \
     if (BM == 256) { if (trans_b) FX_ROWS_WALK(TT, false) else FX_ROWS_WALK(TT, true) }                   \
@@ -414,7 +426,7 @@ extern "C" int fx_grouped_gemm_rows_glu(const void* A, int64_t lda, const void* 
     if (!aligned16(A) || !aligned16(B) || !aligned16(P1) || !aligned16(P2) || !aligned16(act) || (lda & 7) || (ldb & 7) ||
         (ldp & 7) || (ldact & 7) || (K & 63) || (Nh & 7) || (b_expert_stride & 7) || (b2_delta & 7))
         FX_FAIL("fx_grouped_gemm_rows_glu: needs K %% 64 == 0, N %% 8 == 0, strides %% 8 == 0 and 16-byte aligned operands");
-    if (a_row_map && (a_rows <= 0 || (uint64_t)a_rows * (uint64_t)lda * 2u >= (1ull << 32)))
+    if (a_row_map && (a_rows <= 0 || a_rows > 0x7fffffff || (uint64_t)a_rows * (uint64_t)lda * 2u >= (1ull << 32)))
         FX_FAIL("fx_grouped_gemm_rows_glu: a gathered A must have a_rows > 0 and stay below 4 GB");
     GroupedWs w = split_ws(ws, E);
     const int BM = rows_bm(total_rows, E);
@@ -432,7 +444,8 @@ extern "C" int fx_grouped_gemm_rows_glu(const void* A, int64_t lda, const void* 
         kern<<<dim3(max_tiles * (unsigned)tiles_n), WM_ * WN_ * 64, lds, stream>>>(                       \
             reinterpret_cast<const TT*>(A), lda, reinterpret_cast<const TT*>(B), ldb, b_expert_stride,    \
             b2_delta, reinterpret_cast<TT*>(P1), reinterpret_cast<TT*>(P2), ldp, reinterpret_cast<TT*>(act), \
-            ldact, w.ntiles, w.offsets, w.tiles, Nh, K, gate_first, tiles_n, a_row_map);                  \
+            ldact, w.ntiles, w.offsets, w.tiles, Nh, K, gate_first, tiles_n, a_row_map, (int)a_rows, E,   \
+            (int)max_tiles);                                                                              \
     }
     // 128-row tiles: 128 x 256 (128 columns of each half) with 32-wide K-steps, two workgroups per CU
 #define FX_GLU_T(TT)                                                                                      \
@@ -458,8 +471,8 @@ extern "C" int fx_grouped_gemm_wgrad(const void* A, int64_t lda, const void* B, 
     if (!aligned16(A) || !aligned16(B) || (lda & 7) || (ldb & 7) || (M & 7) || (N & 7))
         FX_FAIL("fx_grouped_gemm_wgrad: operands must be 16-byte aligned with M and N multiples of 8");
     GroupedWs w = split_ws(ws, E);
-    if (counts) {    // only the row offsets of the plan are used here: any tile height serves
-        grouped_plan_kernel<<<1, 256, 0, stream>>>(counts, E, 128, w.ntiles, w.offsets, w.tiles);
+    if (counts) {    // only the row offsets are used here; the plan is the one every entry point writes for this shape
+        grouped_plan_kernel<<<1, 256, 0, stream>>>(counts, E, rows_bm(total_rows, E), w.ntiles, w.offsets, w.tiles);
         FX_CHECK_LAUNCH("fx_grouped_gemm_wgrad(plan)");
     }
     constexpr int BM = 256, BN = 256;
@@ -472,7 +485,8 @@ extern "C" int fx_grouped_gemm_wgrad(const void* A, int64_t lda, const void* B, 
         const unsigned grid_w = grid.x < (unsigned)walk_grid() ? grid.x : (unsigned)walk_grid();          \
         kern<<<dim3(grid_w), 2 * 4 * 64, kWalkLdsBytes, stream>>>(                                        \
             reinterpret_cast<const TT*>(A), lda, reinterpret_cast<const TT*>(B), ldb, reinterpret_cast<TG*>(G), ldg, \
-            g_expert_stride, w.offsets, M, N, alpha, beta, tiles_n, tiles_m * tiles_n, (int)grid.x);      \
+            g_expert_stride, w.ntiles, w.offsets, M, N, alpha, beta, tiles_n, tiles_m * tiles_n,          \
+            (int)grid.x, E);                                                                              \
     }
     if (dt == DT_BF16 && g_dt == DT_BF16) FX_WG_WALK(bf16, bf16)
     else if (dt == DT_BF16) FX_WG_WALK(bf16, float)

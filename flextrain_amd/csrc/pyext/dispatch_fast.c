@@ -13,6 +13,7 @@
  * the library and its per-context caches.  Plain C, no dependency beyond the CPython headers. */
 #define PY_SSIZE_T_CLEAN
 #include <Python.h>
+#include <limits.h>
 #include <stddef.h>
 #include <stdint.h>
 
@@ -57,14 +58,35 @@ static PyObject* fast_matmul(PyObject* self, PyObject* const* args, Py_ssize_t n
     intptr_t p[24];
     double r[2] = {0.0, 0.0};
     for (int i = 0; i < 24; ++i) {
+        /* stop at the first argument that does not convert: no C-API call may follow a set exception */
         switch (kKinds[i]) {
-            case AS_PTR: p[i] = (intptr_t)PyLong_AsVoidPtr(args[i]); break;
-            case AS_INT: p[i] = (intptr_t)PyLong_AsLong(args[i]); break;
-            case AS_SIZE: p[i] = (intptr_t)PyLong_AsSize_t(args[i]); break;
-            default: r[i - 22] = PyFloat_AsDouble(args[i]); p[i] = 0; break;
+            case AS_PTR:
+                p[i] = (intptr_t)PyLong_AsVoidPtr(args[i]);
+                if (p[i] == 0 && PyErr_Occurred()) return NULL;
+                break;
+            case AS_INT: {
+                const long v = PyLong_AsLong(args[i]);
+                if (v == -1 && PyErr_Occurred()) return NULL;
+                if (v < INT_MIN || v > INT_MAX) {       /* the dispatcher takes C ints: never truncate silently */
+                    PyErr_Format(PyExc_OverflowError, "matmul_fast: argument %d (%ld) does not fit a C int", i, v);
+                    return NULL;
+                }
+                p[i] = (intptr_t)v;
+                break;
+            }
+            case AS_SIZE: {
+                const size_t v = PyLong_AsSize_t(args[i]);
+                if (v == (size_t)-1 && PyErr_Occurred()) return NULL;
+                p[i] = (intptr_t)v;
+                break;
+            }
+            default:
+                r[i - 22] = PyFloat_AsDouble(args[i]);
+                if (r[i - 22] == -1.0 && PyErr_Occurred()) return NULL;
+                p[i] = 0;
+                break;
         }
     }
-    if (PyErr_Occurred()) return NULL;      /* one of the conversions failed */
     if (p[0] == 0) {
         PyErr_SetString(PyExc_ValueError, "matmul_fast: the dispatcher context is null");
         return NULL;

@@ -344,6 +344,14 @@ def ring_optimizer_step(buffers: LayerRingBuffers, streams: StreamBundle, events
             streams.synchronize_all()
 
     inb, comp, outb = streams.inbound, streams.compute, streams.outbound
+    # The first fetches overwrite the parameter and gradient rings and the activation ring that now
+    # serves as optimizer state, and read host gradients the backward pass offloaded: they must come
+    # after everything already enqueued on the compute stream (last backward kernels) and on the
+    # outbound stream (gradient offloads).  Device-side order only; the host does not wait.
+    for producer in (comp, outb):
+        fence = torch.cuda.Event()
+        fence.record(producer)
+        inb.wait_event(fence)
     for i in range(min(N_P, L)):
         buffers.fetch_layer_params(i, i, skip_frozen=True, stream=inb)
         events.weight_inbound.record_on(i, inb)

@@ -91,7 +91,18 @@ class CublasLtDispatcher:
         self.bf16 = torch.bfloat16
         self.total_python_ns = 0
         self._ctx_int = int(self.ctx) if self.ctx is not None else 0
-        self._fast = _bind_fast()
+        self._fast = self._bind_on_first_fast_call   # ``matmul`` (ctypes) works without the C extension
+
+    def _bind_on_first_fast_call(self, *args):
+        """Stands in for the C entry until it is first needed; from then on ``self._fast`` IS the C
+        function.  A missing extension is reported here, where it is needed, and not by the constructor."""
+        try:
+            self._fast = _bind_fast()
+        except ImportError as err:
+            raise ImportError("flextrain_amd._dispatch_fast is not built for this interpreter "
+                              "(make -C flextrain_amd/csrc PYTHON=<this python>); the validating "
+                              "matmul() path does not need it") from err
+        return self._fast(*args)
 
     def __del__(self):
         if getattr(self, "ctx", None):

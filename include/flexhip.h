@@ -265,8 +265,13 @@ int fx_softcap_bwd(void* dz, const void* gate, int64_t rows, int V, int64_t row_
 size_t fx_grouped_ws_bytes(int E, int64_t total_rows);
 
 /* Row offsets and tile list of one routing, made once and shared by several grouped launches: a
- * grouped entry point called with counts == NULL takes the plan its workspace already holds (same E
- * and total_rows) instead of making it again.  With the per-expert loop of
+ * grouped entry point called with counts == NULL takes the plan its workspace already holds instead
+ * of making it again.  Only a plan written by fx_grouped_plan, or by a grouped entry point that was
+ * given counts, for the SAME E and total_rows may be reused that way (every entry point writes the
+ * same plan for a given shape).  The plan records the E and the tile height it was made for; a
+ * launch that finds another E or tile height there does nothing, and no launch walks more tiles
+ * than total_rows and E allow, so a stale or unplanned workspace cannot send a kernel out of
+ * bounds, but its output is then left unwritten.  With the per-expert loop of
  * flextrain/ops/full_moe.py:428-626 in mind: the counts are read once per pass over the experts,
  * not once per GEMM. */
 int fx_grouped_plan(const int32_t* counts, int E, int64_t total_rows, void* ws, size_t ws_bytes, hipStream_t stream);
@@ -301,7 +306,9 @@ int fx_grouped_gemm_wgrad(const void* A, int64_t lda, const void* B, int64_t ldb
  * product is row a_row_map[r] of A, which then is the UNSORTED (a_rows, K) activation matrix: the
  * tile loads gather the rows, and the scatter launch of flextrain/ops/full_moe.py:131-141 with its
  * expert-sorted copy of the activations is not needed for this product.  a_rows * lda * 2 bytes
- * must stay below 4 GB.  Without a map A is the expert-sorted (total_rows, K) matrix. */
+ * must stay below 4 GB; map entries are clamped to [0, a_rows), so a map that is not a permutation
+ * gives wrong rows, never an access outside A.  Without a map A is the expert-sorted
+ * (total_rows, K) matrix. */
 int fx_grouped_gemm_rows_glu(const void* A, int64_t lda, const void* B, int64_t ldb, int64_t b_expert_stride,
                              int trans_b, int64_t b2_delta, void* P1, void* P2, int64_t ldp, void* act,
                              int64_t ldact, const int32_t* counts, int E, int64_t total_rows, int Nh, int K,

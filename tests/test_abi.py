@@ -60,7 +60,36 @@ def test_fast_call_extension_loads_and_keeps_the_reference_conventions():
     bad[2] = "not a number"
     with pytest.raises(TypeError):
         fast(*bad)
+    # a dimension that does not fit a C int is refused, not truncated; several bad arguments at
+    # once report the first one (no conversion runs after an exception is set)
+    big = list(null_ctx)
+    big[0], big[2] = 1, 1 << 31
+    with pytest.raises(OverflowError):
+        fast(*big)
+    big[3] = "x"
+    with pytest.raises(OverflowError):
+        fast(*big)
+    two_bad = list(null_ctx)
+    two_bad[2], two_bad[22] = "x", "y"
+    with pytest.raises(TypeError):
+        fast(*two_bad)
     # the module-level name of the reference's raw entry resolves to the same C function
     with pytest.raises(TypeError):
         md.matmul_fast(1)
     assert md.matmul_fast is fast
+
+
+def test_dispatcher_constructs_without_the_fast_call_extension(monkeypatch):
+    """The constructor does not need the C extension; only the first fast call does, and says so."""
+    import pytest
+
+    from flextrain_amd import matmul_dispatcher as md
+
+    def missing():
+        raise ImportError("no module named _dispatch_fast")
+
+    monkeypatch.setattr(md, "_bind_fast", missing)
+    disp = md.CublasLtDispatcher()
+    assert disp.get_stats()["matmuls_called"] == 0
+    with pytest.raises(ImportError, match="not built"):
+        disp._fast(0)

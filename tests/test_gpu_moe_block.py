@@ -322,3 +322,53 @@ def test_walking_kernels_fp16_and_int64_row_sources(dev):
     src32 = moe_ops.flextrain_moe_row_sources(mapping.to(torch.int32))
     src64 = moe_ops.flextrain_moe_row_sources(mapping.to(torch.int64))
     assert torch.equal(src32, src64)
+
+
+def test_stale_or_foreign_plan_is_not_consumed(dev):
+    """A grouped launch given no counts takes the plan in its workspace.  Through the raw C ABI: a
+    workspace that was never planned, and one planned for another expert count, leave the output
+    untouched instead of sending the kernel through garbage tile lists; a gathered up-projection whose
+    row map holds out-of-range entries stays inside the source matrix."""
+    from flextrain_amd._lib import dtype_enum, lib, ptr, stream_ptr
+    from flextrain_amd.ops.grouped import GroupedPlan, flextrain_grouped_gemm_rows_glu
+
+    g = gen(808)
+    E, TK, K, N = 4, 2400, 128, 256           # 600 rows per expert: the walking 256-row kernels
+    counts = torch.full((E,), TK // E, dtype=torch.int32, device=dev)
+    A = randn(g, TK, K, std=0.5).to(dev)
+    W = randn(g, E, N, K, std=0.1).to(dev)
+    L = lib()
+    nbytes = int(L.fx_grouped_ws_bytes(E, TK))
+
+    def raw_rows(ws, counts_ptr, D):
+        rc = L.fx_grouped_gemm_rows(ptr(A), K, ptr(W), K, N * K, 1, None, 0, ptr(D), N, counts_ptr, E, TK, N, K, 1.0, 0.0,
+                                    dtype_enum(torch.bfloat16), ptr(ws), nbytes, stream_ptr(dev))
+        assert rc == 0
+        torch.cuda.synchronize()
+
+    want = torch.empty(TK, N, dtype=torch.bfloat16, device=dev)
+    ws_good = torch.zeros(nbytes // 4, dtype=torch.int32, device=dev)
+    raw_rows(ws_good, counts.data_ptr(), want)
+    again = torch.full_like(want, 7.0)
+    raw_rows(ws_good, None, again)                        # the plan the first call left: same bits
+    assert torch.equal(again, want)
+    for ws in (torch.zeros(nbytes // 4, dtype=torch.int32, device=dev),
+               torch.full((nbytes // 4,), 0x7fffffff, dtype=torch.int32, device=dev),
+               GroupedPlan(torch.full((E + 1,), 100, dtype=torch.int32, device=dev), E + 1, TK, dev).ws[:nbytes // 4].clone()):
+        D = torch.full((TK, N), 7.0, dtype=torch.bfloat16, device=dev)
+        raw_rows(ws, None, D)
+        assert bool((D == 7.0).all())
+    # row map with entries outside [0, rows of x): clamped, finite results, rows with valid entries exact
+    T, F = 300, 64
+    x = randn(g, T, K, std=0.5).to(dev)
+    Wg = randn(g, E, 2 * F, K, std=0.1).to(dev)
+    src = torch.randint(0, T, (TK,), generator=g).to(torch.int32)
+    src[::7] = 1 << 30
+    src[3::11] = -5
+    pre = torch.empty(TK, 2 * F, dtype=torch.bfloat16, device=dev)
+    act = torch.empty(TK, F, dtype=torch.bfloat16, device=dev)
+    flextrain_grouped_gemm_rows_glu(x, Wg, counts, pre, act, row_sources=src.to(dev))
+    clamped = src.clamp(0, T - 1).long()
+    pre2, act2 = torch.empty_like(pre), torch.empty_like(act)
+    flextrain_grouped_gemm_rows_glu(x, Wg, counts, pre2, act2, row_sources=clamped.to(torch.int32).to(dev))
+    assert torch.equal(pre, pre2) and torch.equal(act, act2) and bool(torch.isfinite(pre.float()).all())
