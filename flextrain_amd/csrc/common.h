@@ -93,6 +93,32 @@ FX_DEV float glu_fwd_elem(float x1, float x3) {
     }
 }
 
+// Backward of the expert SwiGLU for one element (flextrain/ops/_kernels/moe.py:118-145, and the
+// pre-scaled variant :189-215), shared by the row kernel and the fused dgrad epilogue so that both
+// give the same bits: x3 = value, x1 = gate, d = upstream gradient of the activation, w = the row's
+// router weight.  Returns the element's term of the router-weight gradient.
+FX_DEV float precise_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+template <bool PRESCALED>
+FX_DEV float moe_swiglu_bwd_elem(float x3, float x1, float d, float w, float w_inv, float& dx3, float& dx1, float& act) {
+    const float s = precise_sigmoid(x1);
+    const float silu = x1 * s;
+    const float un = silu * x3;
+    const float ds = s + silu * (1.0f - s);
+    if (PRESCALED) {
+        act = un;
+        dx3 = d * silu;
+        dx1 = d * x3 * ds;
+        return (d * w_inv) * un;
+    } else {
+        act = un * w;
+        const float dsc = d * w;
+        dx3 = dsc * silu;
+        dx1 = dsc * x3 * ds;
+        return d * un;
+    }
+}
+
 // ---------------------------------------------------------------------------
 // Reductions.  `W` lanes (power of two, <= 64) that are contiguous in the wave
 // cooperate; every lane of the group ends with the group's sum.

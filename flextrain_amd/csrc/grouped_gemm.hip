@@ -239,6 +239,163 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void grouped_rows_walk_kern
     }
 }
 
+// ---------------------------------------------------------------- dgrad through w_down with the SwiGLU backward in its epilogue
+// Steps (a) and (b) of the expert backward (flextrain/ops/full_moe.py:589-600) in one launch:
+//   dx_act[r, f] = sum_k dy[r, k] * w_down[e][k, f]                      (rounded to T, never stored)
+//   s = sigmoid(gate), silu = gate * s                                   (x_up[r] = [value (F) | gate (F)])
+//   dx_up[r, f]     = dx_act * w_r * silu                                (gradient of the value half)
+//   dx_up[r, F + f] = dx_act * w_r * value * (s + silu * (1 - s))        (gradient of the gate half)
+//   fwd_act[r, f]   = silu * value * w_r
+//   dprob[r]        = sum_f dx_act * silu * value
+// computed from the ROUNDED dx_act with the element function of the separate kernel
+// (moe_swiglu_bwd_elem), so dx_up and fwd_act carry the bits of the two-launch sequence.  The row
+// sum crosses column tiles: each wave writes the sum over its own 64 columns to
+// PART[r * part_pitch + column_tile * WAVES_N + wave_column] (8-lane tree in a fixed order) and
+// dprob_reduce_kernel adds a row's slots in ascending order: no atomics, the same bits every run.
+template <typename T, typename TW, int WM, int WN, bool LOADS_LAND>
+FX_DEV void epilogue_swiglu_bwd(f32x16_t (&acc)[WM / 32][WN / 32], const T* __restrict__ XUP, int64_t ldx,
+                                const TW* __restrict__ SRW, T* __restrict__ DXUP, int64_t lddx, T* __restrict__ ACT,
+                                int64_t ldact, float* __restrict__ PART, int part_pitch, int part_slot, int row_base,
+                                int col_base, int rows, int F, T* smem, int wave, int lane) {
+    constexpr int TM = WM / 32, TN = WN / 32;
+    constexpr int PITCH = WN + 4;
+    constexpr int GROUPS = WN / 8;
+    constexpr int PER_LANE = 32 * GROUPS / 64;
+    static_assert(GROUPS == 8, "the row sum below reduces over the 8 lanes that share a staged row");
+    typedef typename VecOf<T>::type Pack;
+    static_assert(VecOf<T>::N == 8, "2-byte element types only");
+    float* stage = reinterpret_cast<float*>(smem) + wave * 32 * PITCH;
+    // A band's x_up packs and router weights are requested before the band is staged and used after
+    // it is read back (one register set: a second one in flight spills).
+    Pack px3[1][PER_LANE], px1[1][PER_LANE];
+    float wrow[1][PER_LANE];
+    auto request = [&](int band, int set) {
+#pragma unroll
+        for (int t = 0; t < PER_LANE; ++t) {
+            const int id = t * 64 + lane;
+            const int row = row_base + band * 32 + id / GROUPS, col = col_base + (id % GROUPS) * 8;
+            if (row < rows && col < F) {
+                const T* xr = XUP + (int64_t)row * ldx + col;
+                px3[set][t] = *reinterpret_cast<const Pack*>(xr);
+                px1[set][t] = *reinterpret_cast<const Pack*>(xr + F);
+                wrow[set][t] = (float)SRW[row];
+            }
+        }
+    };
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        request(i, 0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const f32x4_t q = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+                *reinterpret_cast<f32x4_t*>(stage + (lane & 31) * PITCH + j * 32 + 8 * g + 4 * (lane >> 5)) = q;
+            }
+        if (LOADS_LAND && i == TM - 1) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        // a wave reads back only what it wrote itself; its LDS accesses complete in order
+#pragma unroll
+        for (int t = 0; t < PER_LANE; ++t) {
+            const int id = t * 64 + lane;
+            const int rr = id / GROUPS, cg = id % GROUPS;
+            const int row = row_base + i * 32 + rr, col = col_base + cg * 8;
+            float part = 0.f;
+            if (row < rows && col < F) {
+                const float* src = stage + rr * PITCH + cg * 8;
+                const f32x4_t lo = *reinterpret_cast<const f32x4_t*>(src), hi = *reinterpret_cast<const f32x4_t*>(src + 4);
+                const float w = wrow[0][t];
+                float g3[8], g1[8], a[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float d = (float)(T)(e < 4 ? lo[e] : hi[e - 4]);      // dx_act as the separate GEMM would have stored it
+                    part += moe_swiglu_bwd_elem<false>((float)px3[0][t][e], (float)px1[0][t][e], d, w, 0.f, g3[e],
+                                                       g1[e], a[e]);
+                }
+                T* dst = DXUP + (int64_t)row * lddx + col;
+                store_f32<T, 8>(dst, g3);
+                store_f32<T, 8>(dst + F, g1);
+                if (ACT != nullptr) store_f32<T, 8>(ACT + (int64_t)row * ldact + col, a);
+            }
+            // the 8 lanes that share a staged row differ in their low three bits
+            part += __shfl_xor(part, 1, 64);
+            part += __shfl_xor(part, 2, 64);
+            part += __shfl_xor(part, 4, 64);
+            if (cg == 0 && row < rows) PART[(int64_t)row * part_pitch + part_slot] = part;
+        }
+    }
+}
+
+template <typename T, typename TW, int BM, int BN, int WAVES_M, int WAVES_N, bool B_MN>
+__global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void grouped_rows_swiglu_bwd_walk_kernel(
+    const T* __restrict__ A, int64_t lda, const T* __restrict__ B, int64_t ldb, int64_t b_expert_stride,
+    const T* __restrict__ XUP, int64_t ldx, const TW* __restrict__ SRW, T* __restrict__ DXUP, int64_t lddx,
+    T* __restrict__ ACT, int64_t ldact, float* __restrict__ PART, const int32_t* __restrict__ NTILES,
+    const int32_t* __restrict__ OFFSETS, const int32_t* __restrict__ TILES, int F, int K, int tiles_n, int E,
+    int max_tiles) {
+    static_assert((BM + BN) * GEMM_BK * sizeof(T) == 64 * 1024, "the LDS plan assumes 64 KB stages");
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T* smem = reinterpret_cast<T*>(smem_raw);
+    constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+    const int total = plan_total(NTILES, E, BM, tiles_n, max_tiles);
+    int pid = blockIdx.x;
+    if (pid >= total) return;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    struct Tile { int m0, tn, rows, e; int64_t row0; };
+    auto lookup = [&](int id) {
+        const int p = xcd_band(id, total);
+        const int tile = p / tiles_n;
+        Tile t;
+        t.tn = p % tiles_n;
+        t.e = TILES[2 * tile];
+        t.m0 = TILES[2 * tile + 1];
+        t.row0 = OFFSETS[t.e];
+        t.rows = OFFSETS[t.e + 1] - OFFSETS[t.e];
+        return t;
+    };
+    auto view_a = [&](const Tile& t) { return OperandView<T>{A + t.row0 * lda, lda, t.rows, t.m0}; };
+    auto view_b = [&](const Tile& t) { return OperandView<T>{B + (int64_t)t.e * b_expert_stride, ldb, F, t.tn * BN}; };
+    MainLoop2<T, BM, BN, WAVES_M, WAVES_N, false, B_MN> loop;
+    Tile cur = lookup(pid);
+    OperandView<T> a = view_a(cur), b = view_b(cur);
+    loop.begin(a, b, K, WalkLds<T>::buf0(smem));
+    bool landed = false;
+    const int part_pitch = tiles_n * WAVES_N;
+    for (;;) {
+        const int npid = pid + (int)gridDim.x;
+        const bool more = npid < total;
+        Tile nxt = cur;
+        if (more) nxt = lookup(npid);
+        f32x16_t acc[WM / 32][WN / 32];
+        loop.finish(a, b, K, WalkLds<T>::buf0(smem), WalkLds<T>::buf1(smem), acc, landed);
+        const OperandView<T> a2 = view_a(nxt), b2 = view_b(nxt);
+        if (more) loop.begin(a2, b2, K, WalkLds<T>::buf0(smem));
+        epilogue_swiglu_bwd<T, TW, WM, WN, true>(
+            acc, XUP + cur.row0 * ldx, ldx, SRW + cur.row0, DXUP + cur.row0 * lddx, lddx,
+            ACT != nullptr ? ACT + cur.row0 * ldact : nullptr, ldact, PART + cur.row0 * part_pitch, part_pitch,
+            cur.tn * WAVES_N + wave % WAVES_N, cur.m0 + (wave / WAVES_N) * WM, cur.tn * BN + (wave % WAVES_N) * WN, cur.rows, F,
+            WalkLds<T>::epi(smem), wave, lane);
+        if (!more) break;
+        __syncthreads();
+        landed = true;
+        cur = nxt;
+        a = a2;
+        b = b2;
+        pid = npid;
+    }
+}
+
+// dprob[r] = sum of a row's column-slot partial sums, slots ascending.
+template <typename TDW>
+__global__ __launch_bounds__(256) void dprob_reduce_kernel(const float* __restrict__ PART, int pitch, TDW* __restrict__ DW,
+                                                           int64_t rows) {
+    const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (r >= rows) return;
+    float s = 0.f;
+    for (int p = 0; p < pitch; ++p) s += PART[r * pitch + p];
+    DW[r] = (TDW)s;
+}
+
 template <typename T, typename TG, int BM, int BN, int WAVES_M, int WAVES_N>
 __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void grouped_wgrad_walk_kernel(
     const T* __restrict__ A, int64_t lda, const T* __restrict__ B, int64_t ldb, TG* G, int64_t ldg,
@@ -493,5 +650,70 @@ extern "C" int fx_grouped_gemm_wgrad(const void* A, int64_t lda, const void* B, 
     else FX_WG_WALK(f16, f16)
 #undef FX_WG_WALK
     FX_CHECK_LAUNCH("fx_grouped_gemm_wgrad");
+    return 0;
+}
+
+extern "C" int fx_grouped_rows_tile_height(int E, int64_t total_rows) { return rows_bm(total_rows, E); }
+
+extern "C" size_t fx_grouped_swiglu_bwd_ws_bytes(int64_t total_rows, int F) {
+    if (total_rows < 0 || F <= 0) return 0;
+    return sizeof(float) * (size_t)total_rows * (size_t)(cdiv_i(F, 256) * 4);
+}
+
+extern "C" int fx_grouped_gemm_rows_swiglu_bwd(const void* dy, int64_t lddy, const void* w_down, int64_t ldb,
+                                               int64_t b_expert_stride, int trans_b, const void* x_up, int64_t ldx,
+                                               const void* srw, int srw_dt, void* dx_up, int64_t lddx, void* fwd_act,
+                                               int64_t ldact, void* dprob, int dprob_dt, const int32_t* counts, int E,
+                                               int64_t total_rows, int F, int K, int dt, void* ws, size_t ws_bytes,
+                                               void* part_ws, size_t part_ws_bytes, hipStream_t stream) {
+    if (E <= 0 || total_rows < 0 || F <= 0 || K <= 0) FX_FAIL("fx_grouped_gemm_rows_swiglu_bwd: bad shape");
+    if (total_rows == 0) return 0;
+    if (!dy || !w_down || !x_up || !srw || !dx_up || !dprob) FX_FAIL("fx_grouped_gemm_rows_swiglu_bwd: null pointer");
+    if (!ws || ws_bytes < fx_grouped_ws_bytes(E, total_rows)) FX_FAIL("fx_grouped_gemm_rows_swiglu_bwd: workspace too small");
+    if (!part_ws || part_ws_bytes < fx_grouped_swiglu_bwd_ws_bytes(total_rows, F) || !aligned16(part_ws))
+        FX_FAIL("fx_grouped_gemm_rows_swiglu_bwd: partial-sum workspace missing, misaligned or too small");
+    if (dt != DT_BF16 && dt != DT_F16) FX_FAIL("fx_grouped_gemm_rows_swiglu_bwd: bf16 or fp16 only");
+    if (srw_dt != dt && srw_dt != DT_F32) FX_FAIL("fx_grouped_gemm_rows_swiglu_bwd: router weights must have the activations' dtype or be fp32");
+    if (dprob_dt != dt && dprob_dt != DT_F32) FX_FAIL("fx_grouped_gemm_rows_swiglu_bwd: dprob must have the activations' dtype or be fp32");
+    if (rows_bm(total_rows, E) != 256) FX_FAIL("fx_grouped_gemm_rows_swiglu_bwd: needs 256-row tiles (at least 384 rows per expert on average); run the GEMM and fx_swiglu_moe_bwd separately");
+    if (lddy >= (1 << 23) || ldb >= (1 << 23)) FX_FAIL("fx_grouped_gemm_rows_swiglu_bwd: leading dimensions must be below 2^23 elements");
+    if (!aligned16(dy) || !aligned16(w_down) || !aligned16(x_up) || !aligned16(dx_up) || (fwd_act && !aligned16(fwd_act)) ||
+        (lddy & 7) || (ldb & 7) || (ldx & 7) || (lddx & 7) || (fwd_act && (ldact & 7)) || (K & 7) || (F & 7) ||
+        (b_expert_stride & 7))
+        FX_FAIL("fx_grouped_gemm_rows_swiglu_bwd: operands must be 16-byte aligned with K, F and every row stride a multiple of 8");
+    if (ldx < 2 * (int64_t)F || lddx < 2 * (int64_t)F || (fwd_act && ldact < F)) FX_FAIL("fx_grouped_gemm_rows_swiglu_bwd: x_up / dx_up rows hold 2 F elements, fwd_act rows F");
+    GroupedWs w = split_ws(ws, E);
+    constexpr int BM = 256;
+    if (counts) {
+        grouped_plan_kernel<<<1, 256, 0, stream>>>(counts, E, BM, w.ntiles, w.offsets, w.tiles);
+        FX_CHECK_LAUNCH("fx_grouped_gemm_rows_swiglu_bwd(plan)");
+    }
+    const unsigned max_tiles = (unsigned)(total_rows / BM + E);
+    const int tiles_n = cdiv_i(F, 256);
+    const unsigned most = max_tiles * (unsigned)tiles_n;
+    const unsigned grid = most < (unsigned)walk_grid() ? most : (unsigned)walk_grid();
+#define FX_SWB(TT, TW, BMN)                                                                               \
+    {                                                                                                     \
+        auto kern = grouped_rows_swiglu_bwd_walk_kernel<TT, TW, 256, 256, 2, 4, BMN>;                     \
+        FX_ENSURE_DYNAMIC_LDS(kern, kWalkLdsBytes);                                                       \
+        kern<<<dim3(grid), 512, kWalkLdsBytes, stream>>>(                                                 \
+            reinterpret_cast<const TT*>(dy), lddy, reinterpret_cast<const TT*>(w_down), ldb, b_expert_stride, \
+            reinterpret_cast<const TT*>(x_up), ldx, reinterpret_cast<const TW*>(srw), reinterpret_cast<TT*>(dx_up), \
+            lddx, reinterpret_cast<TT*>(fwd_act), ldact, reinterpret_cast<float*>(part_ws), w.ntiles, w.offsets, \
+            w.tiles, F, K, tiles_n, E, (int)max_tiles);                                                   \
+    }
+#define FX_SWB_T(TT)                                                                                      \
+    if (srw_dt == DT_F32) { if (trans_b) FX_SWB(TT, float, false) else FX_SWB(TT, float, true) }          \
+    else { if (trans_b) FX_SWB(TT, TT, false) else FX_SWB(TT, TT, true) }
+    if (dt == DT_BF16) { FX_SWB_T(bf16) } else { FX_SWB_T(f16) }
+#undef FX_SWB_T
+#undef FX_SWB
+    FX_CHECK_LAUNCH("fx_grouped_gemm_rows_swiglu_bwd");
+    const unsigned rgrid = (unsigned)((total_rows + 255) / 256);
+    const int pitch = tiles_n * 4;
+    if (dprob_dt == DT_F32) dprob_reduce_kernel<float><<<rgrid, 256, 0, stream>>>(reinterpret_cast<const float*>(part_ws), pitch, reinterpret_cast<float*>(dprob), total_rows);
+    else if (dt == DT_BF16) dprob_reduce_kernel<bf16><<<rgrid, 256, 0, stream>>>(reinterpret_cast<const float*>(part_ws), pitch, reinterpret_cast<bf16*>(dprob), total_rows);
+    else dprob_reduce_kernel<f16><<<rgrid, 256, 0, stream>>>(reinterpret_cast<const float*>(part_ws), pitch, reinterpret_cast<f16*>(dprob), total_rows);
+    FX_CHECK_LAUNCH("fx_grouped_gemm_rows_swiglu_bwd(reduce)");
     return 0;
 }

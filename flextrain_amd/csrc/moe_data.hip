@@ -176,22 +176,7 @@ __global__ __launch_bounds__(256) void swiglu_moe_bwd_kernel(
     const float w_inv = 1.0f / fmaxf(1e-8f, w);
     float dw = 0.f;
     auto elem = [&](float x3, float x1, float d, float& dx3, float& dx1, float& act) {
-        const float s = sigmoidf_(x1);
-        const float silu = x1 * s;
-        const float un = silu * x3;
-        const float ds = s + silu * (1.0f - s);
-        if (PRESCALED) {
-            act = un;
-            dw += (d * w_inv) * un;
-            dx3 = d * silu;
-            dx1 = d * x3 * ds;
-        } else {
-            act = un * w;
-            dw += d * un;
-            const float dsc = d * w;
-            dx3 = dsc * silu;
-            dx1 = dsc * x3 * ds;
-        }
+        dw += moe_swiglu_bwd_elem<PRESCALED>(x3, x1, d, w, w_inv, dx3, dx1, act);
     };
     if (vec) {
         for (int c = lane * 8; c < F; c += 512) {

@@ -20,8 +20,10 @@ from .ops.grouped import (
     GroupedPlan,
     flextrain_grouped_gemm_rows,
     flextrain_grouped_gemm_rows_glu,
+    flextrain_grouped_gemm_rows_swiglu_bwd,
     flextrain_grouped_gemm_wgrad,
     grouped_glu_supported,
+    grouped_swiglu_bwd_supported,
 )
 from .ops.moe import (
     flextrain_fused_topk_softmax,
@@ -152,12 +154,17 @@ def swiglu_expert_loop_bwd(scattered_upstream, scattered_x, x_preact_buf, srw, d
     # second stream only take CUs from the first (measured at 8192 tokens x 128 experts: weight
     # gradients on the secondary stream 2.06 ms against 2.01 ms for the same work on one stream).
     with torch.cuda.stream(primary_stream):
-        dx_act = torch.empty((TK, expert_dim), dtype=scattered_upstream.dtype, device=scattered_upstream.device)
-        fwd_act = torch.empty_like(dx_act)
+        fwd_act = torch.empty((TK, expert_dim), dtype=scattered_upstream.dtype, device=scattered_upstream.device)
         plan = GroupedPlan(counts, w_up.shape[0], TK, scattered_upstream.device)
-        flextrain_grouped_gemm_rows(scattered_upstream, w_down, counts, dx_act, plan=plan)             # (a)
-        flextrain_swiglu_moe_bwd(dx_act, x_preact_buf[:TK], srw[:TK], dx=dx_up_up_grouped[:TK], dw=dprobs[:TK],
-                                 fwd_act=fwd_act)                                                       # (b)
+        dx_up, x_up, rw, dpr = dx_up_up_grouped[:TK], x_preact_buf[:TK], srw[:TK], dprobs[:TK]
+        if grouped_swiglu_bwd_supported(scattered_upstream, w_down, x_up, rw, dx_up, fwd_act, dpr):
+            # (a) + (b) in one launch: dx_act lives only in the dgrad's epilogue
+            flextrain_grouped_gemm_rows_swiglu_bwd(scattered_upstream, w_down, counts, x_up, rw, dx_up, dpr,
+                                                   fwd_act=fwd_act, plan=plan)
+        else:
+            dx_act = torch.empty_like(fwd_act)
+            flextrain_grouped_gemm_rows(scattered_upstream, w_down, counts, dx_act, plan=plan)         # (a)
+            flextrain_swiglu_moe_bwd(dx_act, x_up, rw, dx=dx_up, dw=dpr, fwd_act=fwd_act)               # (b)
         if grads.get("g_down") is not None:
             flextrain_grouped_gemm_wgrad(scattered_upstream, fwd_act, grads["g_down"], counts, plan=plan)   # (c)
         flextrain_grouped_gemm_rows(dx_up_up_grouped[:TK], w_up, counts, dx_pre_grouped[:TK], plan=plan)    # (d)

@@ -159,6 +159,51 @@ def flextrain_grouped_gemm_rows_glu(A, w_up, counts, pre, act, row_sources=None,
     return pre, act
 
 
+def grouped_swiglu_bwd_supported(dy, w_down, x_up, srw, dx_up, fwd_act, dprob):
+    """Whether :func:`flextrain_grouped_gemm_rows_swiglu_bwd` can take these tensors (else the
+    caller runs the dgrad GEMM and ``flextrain_swiglu_moe_bwd`` separately)."""
+    if dy.dtype not in (torch.bfloat16, torch.float16) or w_down.dim() != 3 or not w_down.is_contiguous():
+        return False
+    E, d, F = w_down.shape
+    TK = dy.shape[0]
+    if any(t.dtype != dy.dtype for t in (w_down, x_up, dx_up)) or (fwd_act is not None and fwd_act.dtype != dy.dtype):
+        return False
+    if srw.dtype not in (dy.dtype, torch.float32) or dprob.dtype not in (dy.dtype, torch.float32):
+        return False
+    if not (srw.is_contiguous() and dprob.is_contiguous() and srw.numel() == TK and dprob.numel() == TK):
+        return False
+    two_d = [dy, x_up, dx_up] + ([fwd_act] if fwd_act is not None else [])
+    if any(t.dim() != 2 or t.stride(1) != 1 or t.stride(0) % 8 or t.data_ptr() % 16 or t.shape[0] != TK for t in two_d):
+        return False
+    if dy.shape[1] != d or x_up.shape[1] != 2 * F or dx_up.shape[1] != 2 * F or (fwd_act is not None and fwd_act.shape[1] != F):
+        return False
+    return (d % 8 == 0 and F % 8 == 0 and w_down.data_ptr() % 16 == 0
+            and int(lib().fx_grouped_rows_tile_height(E, TK)) == 256)
+
+
+def flextrain_grouped_gemm_rows_swiglu_bwd(dy, w_down, counts, x_up, srw, dx_up, dprob, fwd_act=None, plan=None):
+    """Expert dgrad through ``w_down (E, d, F)`` with the weighted SwiGLU backward in its epilogue:
+    ``dx_act = dy[rows_e] @ w_down[e]`` is rounded and consumed in registers;
+    ``dx_up (TK, 2F)``, ``fwd_act (TK, F) = act * w`` and ``dprob (TK,) = sum_F dx_act * act`` are
+    written.  ``x_up (TK, 2F)`` is the saved pre-activation ``[value | gate]``, ``srw`` the
+    expert-sorted router weights.  ``dx_up`` / ``fwd_act`` equal, bit for bit, what
+    ``flextrain_grouped_gemm_rows`` + ``flextrain_swiglu_moe_bwd`` give."""
+    if not grouped_swiglu_bwd_supported(dy, w_down, x_up, srw, dx_up, fwd_act, dprob):
+        raise ValueError("unsupported operands for the fused dgrad + SwiGLU backward (see grouped_swiglu_bwd_supported)")
+    E, d, F = w_down.shape
+    TK = dy.shape[0]
+    cptr, ws, nbytes = _plan_or_workspace(plan, counts, E, TK, dy.device)
+    part_bytes = int(lib().fx_grouped_swiglu_bwd_ws_bytes(TK, F))
+    part = torch.empty(part_bytes // 4, dtype=torch.float32, device=dy.device)
+    rc = lib().fx_grouped_gemm_rows_swiglu_bwd(
+        ptr(dy), dy.stride(0), ptr(w_down), F, w_down.stride(0), 0, ptr(x_up), x_up.stride(0), ptr(srw),
+        dtype_enum(srw.dtype), ptr(dx_up), dx_up.stride(0), ptr(fwd_act), fwd_act.stride(0) if fwd_act is not None else 0,
+        ptr(dprob), dtype_enum(dprob.dtype), cptr, E, TK, F, d, dtype_enum(dy.dtype), ptr(ws), nbytes, ptr(part),
+        part_bytes, stream_ptr(dy.device))
+    check(rc, "fx_grouped_gemm_rows_swiglu_bwd")
+    return dx_up, dprob, fwd_act
+
+
 _ACT_ENUM = {"silu": 0, "gelu_tanh": 1}
 
 

@@ -315,6 +315,30 @@ int fx_grouped_gemm_rows_glu(const void* A, int64_t lda, const void* B, int64_t 
                              int gate_first, int dt, void* ws, size_t ws_bytes, const int32_t* a_row_map,
                              int64_t a_rows, hipStream_t stream);
 
+/* Steps (a) and (b) of the expert backward (flextrain/ops/full_moe.py:589-600: the dgrad GEMM through
+ * w_down, then the weighted SwiGLU backward of flextrain/ops/_kernels/moe.py:77-145) as one launch
+ * plus a small reduction: dx_act = dy_e @ op(w_down[e]) is rounded to the storage type in the
+ * epilogue and never stored;
+ *   dx_up[r] = [dx_act * w_r * silu(gate) | dx_act * w_r * value * dsilu(gate)]   (rows of 2 F)
+ *   fwd_act[r] = silu(gate) * value * w_r                                         (rows of F; may be NULL)
+ *   dprob[r] = sum_f dx_act * silu(gate) * value
+ * with x_up[r] = [value (F) | gate (F)] the saved pre-activation and srw[r] = w_r the router weight
+ * of expert-sorted row r.  dx_up and fwd_act carry the bits of fx_grouped_gemm_rows followed by
+ * fx_swiglu_moe_bwd; dprob is summed in a fixed order (per-wave column slots in part_ws, then a
+ * reduction), reproducible from run to run but not in the order of that kernel.
+ * K = d_model, F = expert width; trans_b as fx_grouped_gemm_rows (w_down stored (E, d, F): 0).
+ * part_ws: fx_grouped_swiglu_bwd_ws_bytes(total_rows, F) bytes, 16-byte aligned.
+ * Needs the 256-row tile form (fx_grouped_rows_tile_height(E, total_rows) == 256), K, F and all
+ * row strides multiples of 8. */
+int fx_grouped_rows_tile_height(int E, int64_t total_rows);
+size_t fx_grouped_swiglu_bwd_ws_bytes(int64_t total_rows, int F);
+int fx_grouped_gemm_rows_swiglu_bwd(const void* dy, int64_t lddy, const void* w_down, int64_t ldb,
+                                    int64_t b_expert_stride, int trans_b, const void* x_up, int64_t ldx,
+                                    const void* srw, int srw_dt, void* dx_up, int64_t lddx, void* fwd_act,
+                                    int64_t ldact, void* dprob, int dprob_dt, const int32_t* counts, int E,
+                                    int64_t total_rows, int F, int K, int dt, void* ws, size_t ws_bytes, void* part_ws,
+                                    size_t part_ws_bytes, hipStream_t stream);
+
 /* Gate and up projections of the dense gated FFN with the activation in the epilogue: replaces the
  * two matmuls and the gated-activation launch of flextrain/nn/blocks/ffn_dense.py:130-146.
  *   P1 = A @ op(B1), P2 = A @ op(B2) (both (M, Nh), row stride ldp), act = f(gate) * value

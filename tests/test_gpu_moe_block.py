@@ -372,3 +372,53 @@ def test_stale_or_foreign_plan_is_not_consumed(dev):
     pre2, act2 = torch.empty_like(pre), torch.empty_like(act)
     flextrain_grouped_gemm_rows_glu(x, Wg, counts, pre2, act2, row_sources=clamped.to(torch.int32).to(dev))
     assert torch.equal(pre, pre2) and torch.equal(act, act2) and bool(torch.isfinite(pre.float()).all())
+
+
+@pytest.mark.parametrize("E,TK,d,F", [(4, 2400, 128, 64), (3, 1800, 256, 264), (128, 65536, 2048, 768)])
+@pytest.mark.parametrize("dprob_dtype", [torch.bfloat16, torch.float32])
+def test_fused_dgrad_swiglu_bwd_equals_the_two_launches(dev, E, TK, d, F, dprob_dtype):
+    """Steps (a) + (b) of the expert backward (flextrain/ops/full_moe.py:589-600) as one launch against
+    the dgrad GEMM followed by the SwiGLU-backward kernel: dx_up and the saved activation bit for bit
+    (both evaluate the same element function on the same rounded dx_act), the router-weight gradient
+    within the bf16 tolerance (its fp32 row sum runs in another order), and against the oracle."""
+    from flextrain_amd.ops import moe as moe_ops
+    from flextrain_amd.ops.grouped import (flextrain_grouped_gemm_rows_swiglu_bwd, grouped_swiglu_bwd_supported)
+
+    g = gen(E * 31 + F)
+    counts = _ragged_counts(g, E, TK)
+    dy = randn(g, TK, d, std=0.5)
+    w_down = randn(g, E, d, F, std=0.1)
+    x_up = randn(g, TK, 2 * F)
+    srw = torch.rand(TK, 1, generator=g).to(torch.bfloat16)
+    dyd, wd, xd, sd, cd = dy.to(dev), w_down.to(dev), x_up.to(dev), srw.to(dev), counts.to(dev)
+    # the two launches
+    dx_act = torch.empty(TK, F, dtype=torch.bfloat16, device=dev)
+    flextrain_grouped_gemm_rows(dyd, wd, cd, dx_act)
+    dx_ref = torch.empty(TK, 2 * F, dtype=torch.bfloat16, device=dev)
+    act_ref = torch.empty(TK, F, dtype=torch.bfloat16, device=dev)
+    dw_ref = torch.empty(TK, 1, dtype=dprob_dtype, device=dev)
+    moe_ops.flextrain_swiglu_moe_bwd(dx_act, xd, sd, dx=dx_ref, dw=dw_ref, fwd_act=act_ref)
+    # one launch
+    dx = torch.full_like(dx_ref, 7.0)
+    act = torch.full_like(act_ref, 7.0)
+    dw = torch.full_like(dw_ref, 7.0)
+    assert grouped_swiglu_bwd_supported(dyd, wd, xd, sd, dx, act, dw)
+    flextrain_grouped_gemm_rows_swiglu_bwd(dyd, wd, cd, xd, sd, dx, dw, fwd_act=act)
+    assert torch.equal(dx, dx_ref), f"dx_up differs in {int((dx != dx_ref).sum())} of {dx.numel()} elements"
+    assert torch.equal(act, act_ref)
+    _close_scaled(dw, dw_ref, "router-weight gradient, fused vs two launches")
+    # twice the same bits (fixed summation order)
+    dw2 = torch.empty_like(dw)
+    flextrain_grouped_gemm_rows_swiglu_bwd(dyd, wd, cd, xd, sd, torch.empty_like(dx), dw2, fwd_act=None)
+    assert torch.equal(dw, dw2)
+    # against the oracle on a few experts
+    off = o_moe.expert_offsets(counts)
+    for e in (range(E) if E <= 8 else (0, 2, 127)):
+        a, b = int(off[e]), int(off[e + 1])
+        if a == b:
+            continue
+        dact = (dy[a:b].float() @ w_down[e].float()).to(torch.bfloat16)
+        want_dx, want_dw, want_act = o_moe.swiglu_moe_bwd(dact, x_up[a:b], srw[a:b])
+        _close_scaled(dx[a:b], want_dx, f"dx_up of expert {e}")
+        _close_scaled(act[a:b], want_act, f"saved activation of expert {e}")
+        _close_scaled(dw[a:b].reshape(-1), want_dw.reshape(-1), f"router-weight gradient of expert {e}")
