@@ -35,10 +35,32 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0       # MI355X HBM3E, published
 BF16_PEAK_TFLOPS = 2500.0    # MI355X dense bf16 MFMA, published
 
-# HBM bytes per launch of the SwiGLU backward kernel at the benchmark shape, from the FETCH_SIZE and
-# WRITE_SIZE hardware counters scaled by what they read for a plain copy of known size
-# (profiles/glu_bwd_hbm_traffic_pmc.txt holds the counter values and the commands).
-GLU_BWD_MEASURED_TRAFFIC_BYTES = 1_174_285_231
+# HBM bytes per launch of the SwiGLU backward kernel at the benchmark shape come from the FETCH_SIZE
+# and WRITE_SIZE hardware counters, each scaled by what it reads for a plain copy of known size.  The
+# counter values live in this text summary (with the commands that produced them); the figure is
+# recomputed from it on every run, and is null when the file is missing or does not parse.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "glu_bwd_hbm_traffic_pmc.txt")
+
+
+def _measured_traffic_bytes(path=TRAFFIC_PROFILE):
+    """`key: value` lines of the summary: KiB per dispatch of the calibration copy and of the kernel."""
+    want = ("copy_bytes_each_way", "copy_FETCH_SIZE_KiB", "copy_WRITE_SIZE_KiB", "glu_bwd_FETCH_SIZE_KiB",
+            "glu_bwd_WRITE_SIZE_KiB")
+    vals = {}
+    try:
+        with open(path) as f:
+            for line in f:
+                key, _, rest = line.partition(":")
+                if key.strip() in want:
+                    vals[key.strip()] = float(rest.split()[0].replace(",", ""))
+    except (OSError, ValueError, IndexError):
+        return None
+    if any(k not in vals for k in want) or vals["copy_FETCH_SIZE_KiB"] <= 0 or vals["copy_WRITE_SIZE_KiB"] <= 0:
+        return None
+    copy_kib = vals["copy_bytes_each_way"] / 1024.0
+    read = vals["glu_bwd_FETCH_SIZE_KiB"] * (copy_kib / vals["copy_FETCH_SIZE_KiB"])
+    written = vals["glu_bwd_WRITE_SIZE_KiB"] * (copy_kib / vals["copy_WRITE_SIZE_KiB"])
+    return int(round((read + written) * 1024.0))
 
 METRIC = "per-op HBM GB/s (% of 8 TB/s) + lm_head/MoE GEMM TFLOPS (% bf16 MFMA peak)"
 
@@ -189,6 +211,22 @@ def run_dispatch_overhead(torch, dev, stream):
     st1 = disp.get_stats()
     cpp_us = ((st1["avg_cpp_total_us"] * st1["matmuls_called"] - st0["avg_cpp_total_us"] * st0["matmuls_called"])
               / max(1, st1["matmuls_called"] - st0["matmuls_called"]))
+    # the library's own split of that time (get_stats: key construction, cache look-up, and the enqueue =
+    # current-device query + kernel launch call), over a window of calls of its own
+    import ctypes
+
+    def raw_stats():
+        buf = (ctypes.c_uint64 * 7)()
+        disp._lib.get_stats(disp.ctx, buf)
+        return list(buf)
+
+    r0 = raw_stats()
+    for _ in range(n):
+        fast(*raw)
+    torch.cuda.synchronize()
+    r1 = raw_stats()
+    calls = max(1, r1[1] - r0[1])
+    total_us, key_us, lookup_us, enqueue_us = ((r1[i] - r0[i]) / calls / 1e3 for i in (3, 4, 5, 6))
     us_fast = per_call(lambda: disp.matmul_fast(sp, A, A, D=D))
     us_full = per_call(lambda: disp.matmul(sp, A, A, D=D))
     return [{"op": "disp.host time per dispatcher call (64^3 GEMM, 2000 calls back to back)", "algorithmic": None,
@@ -196,6 +234,9 @@ def run_dispatch_overhead(torch, dev, stream):
              "matmul_ctypes_us": round(us_full, 2), "matmul_fast_method_us": round(us_fast, 2),
              "raw_fast_call_entry_us": round(us_raw, 2), "library_time_per_call_us": round(cpp_us, 2),
              "raw_fast_call_entry_mean_us": round(us_raw_mean, 2),
+             "library_split_us": {"key": round(key_us, 3), "cache_lookup": round(lookup_us, 3),
+                                  "enqueue (device query + launch call)": round(enqueue_us, 3),
+                                  "other (argument checks, clock reads, error query)": round(max(0.0, total_us - key_us - lookup_us - enqueue_us), 3)},
              "raw_entry_overhead_over_library_us": round(max(0.0, us_raw_mean - cpp_us), 2)}]
 
 
@@ -416,18 +457,18 @@ def run_lm_head(torch, dev, stream, rn):
         grads["g_head_proj"] = g_head.t()
         ms = _time_launches(torch, stream, [run], warmup=1, reps=3)
         row = _op_entry(name, 6 * T * d * V, "TFLOP/s", ms)
-        groups = fuse if fuse is not None else max(1, head.cfg.logits_buffer_bytes // chunk_bytes)
+        groups = fuse if fuse is not None else max(1, min(T // chunk, head.cfg.logits_buffer_bytes // chunk_bytes))
         row["logits_buffer_MB"] = round(groups * chunk_bytes / 1e6)
         row["head_gradient"] = str(g_head.dtype).replace("torch.", "")
         rows.append(row)
 
     # The reference's own schedule and gradient type first (one 1024-token logits buffer; torch.addmm
-    # into a compute-dtype accumulator, flextrain/nn/head.py:82-84, :324-331), then the same with the
-    # fp32 accumulator this package also takes, then larger GEMM groups.
+    # into a compute-dtype accumulator, flextrain/nn/head.py:82-84, :324-331: the head's default here
+    # too), then the same with the fp32 accumulator this package also takes, then the opt-in 8-chunk
+    # GEMM groups (a 2.1 GB logits buffer).
     head_row("c3.lm_head fwd+bwd (chunk 1024, one GEMM group per chunk and bf16 dW += as the reference)", 1, g_bf16)
     head_row("c3.lm_head fwd+bwd (chunk 1024, one GEMM group per chunk, fp32 dW +=)", 1, g_store)
-    head_row("c3.lm_head fwd+bwd (chunk 1024 x 2 per GEMM group: the default, fp32 dW +=)", None, g_store)
-    head_row("c3.lm_head fwd+bwd (chunk 1024 x 8 per GEMM group, fp32 dW +=)", 8, g_store)
+    head_row("c3.lm_head fwd+bwd (chunk 1024 x 8 per GEMM group: opt-in, fp32 dW +=)", 8, g_store)
     # the three GEMMs of one micro-chunk, timed alone
     disp = CublasLtDispatcher()
     sp = stream.cuda_stream
@@ -722,7 +763,67 @@ def run_moe(torch, dev, stream, rn):
     ms = _time_launches(torch, stream, [lambda: flextrain_grouped_gemm_wgrad(pre, sx, grads["g_up"], counts)], warmup=2, reps=10)
     rows.append(floor(_op_entry("c5.grouped wgrad g_up [1536,T_e]x[T_e,2048] x128 (+= bf16)", 2 * TK * d * 2 * F, "TFLOP/s", ms),
                       2 * TK * d * 2 * F, 2 * (TK * 2 * F + TK * d + 2 * E * 2 * F * d)))
+    del sx, act, x, dy, out, weights, grads, slot
+    pool.clear()
+    torch.cuda.empty_cache()
+    rows += _moe_reference_microbench(torch, dev, stream, rn)
     return rows
+
+
+def _moe_reference_microbench(torch, dev, stream, rn):
+    """The shape and scope of the reference's own MoE micro-benchmark
+    (external_moe_impl/bench/bench_moe.py:4-13): d 2048, F 512, 256 experts, top-8, 16 K tokens;
+    routed-MLP scope = scatter -> experts -> weighted gather (no router GEMM, no residual) forward,
+    dy -> dx, g_up, g_down backward."""
+    import types
+
+    from flextrain_amd.moe_backend import FlextrainMoEExpertCompute
+    from flextrain_amd.ops.moe import flextrain_fused_topk_softmax
+
+    T, d, E, K, F = 16384, 2048, 256, 8, 512
+    TK = T * K
+    bf = torch.bfloat16
+    x, dy = rn(T, d).to(dev), rn(T, d).to(dev)
+    weights = dict(w_up=(torch.randn(E, 2 * F, d, device=dev) * 0.02).to(bf), w_down=(torch.randn(E, d, F, device=dev) * 0.02).to(bf))
+    grads = dict(g_up=torch.zeros(E, 2 * F, d, dtype=bf, device=dev), g_down=torch.zeros(E, d, F, dtype=bf, device=dev))
+    slot = types.SimpleNamespace(
+        index_mapping=torch.empty(T, K, dtype=torch.int32, device=dev), expert_counts=torch.empty(E, dtype=torch.int32, device=dev),
+        scattered_router_weights=torch.empty(TK, 1, dtype=bf, device=dev), x_up=torch.empty(TK, 2 * F, dtype=bf, device=dev), aux={})
+    logits = torch.randn(T, E, device=dev).to(bf)
+    ids = torch.empty(T, K, dtype=torch.int32, device=dev)
+    probs = torch.empty(T, K, dtype=bf, device=dev)
+    flextrain_fused_topk_softmax(logits, top_k=K, topk_ids_out=ids, topk_weights_out=probs, mode="topk_then_softmax")
+    backend = FlextrainMoEExpertCompute()
+    bufs = {}
+
+    def scratch(shape, dtype):
+        key = (tuple(shape), dtype, sum(1 for k in bufs if k[:2] == (tuple(shape), dtype) and bufs[k][1]))
+        if key not in bufs:
+            bufs[key] = [torch.empty(shape, dtype=dtype, device=dev), False]
+        bufs[key][1] = True
+        return bufs[key][0]
+
+    def release():
+        for v in bufs.values():
+            v[1] = False
+
+    out, dx, extra = torch.empty(T, d, dtype=bf, device=dev), torch.empty(T, d, dtype=bf, device=dev), {}
+    common = dict(slot=slot, chunk_extra=extra, layer_id=0, primary_stream=stream, secondary_stream=None, scratch_fn=scratch)
+
+    def fwd():
+        release()
+        backend.fwd(x, probs, ids, weights, out=out, residual=None, **common)
+
+    def bwd():
+        release()
+        backend.bwd(dy, x, weights, grads, dx=dx, **common)
+        slot.aux.pop("moe_dprobs", None)
+
+    ms_f = _time_launches(torch, stream, [fwd], warmup=2, reps=5)
+    ms_b = _time_launches(torch, stream, [bwd], warmup=2, reps=5)
+    name = "moe_ref.routed MLP, the reference's micro-benchmark shape (16384 tokens, d 2048, F 512, 256 experts, top-8)"
+    return [_op_entry(name + " fwd", 6 * TK * d * F, "TFLOP/s", ms_f), _op_entry(name + " bwd", 12 * TK * d * F, "TFLOP/s", ms_b),
+            _op_entry(name + " fwd+bwd", 18 * TK * d * F, "TFLOP/s", ms_f + ms_b)]
 
 
 def _cpu_model():
@@ -921,7 +1022,7 @@ def main():
     dom_gbps = swiglu_bwd_bytes / (dom_ms * 1e-3) / 1e9
     roofline = {"kernel": "glu_bwd_kernel<bf16, silu>", "bound": "hbm", "achieved": round(dom_gbps, 1),
                 "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(dom_gbps / HBM_PEAK_GBPS, 4),
-                "traffic": GLU_BWD_MEASURED_TRAFFIC_BYTES, "algorithmic_bytes": swiglu_bwd_bytes, "avg_ms": round(dom_ms, 5)}
+                "traffic": _measured_traffic_bytes(), "algorithmic_bytes": swiglu_bwd_bytes, "avg_ms": round(dom_ms, 5)}
     # RoPE rows: timed over >= 100 back-to-back launches that rotate through the buffer sets (every launch
     # reads from HBM).  Then the same launches on ONE buffer set: the cache-resident case (in a layer q
     # and k come straight out of the projection GEMM).
@@ -987,6 +1088,49 @@ def main():
                "sample": f"CPU oracle (PyTorch fp32 formulas) on the first {Ts} of {T} tokens of the same "
                          f"workload, median of {len(times)} runs, {med * 1e3:.1f} ms each"}
 
+    # The MFMA-bound half of the metric: the LM-head logits GEMM of one 1024-token chunk as the kernel
+    # record (flop per launch over its event-timed launch duration), with the whole C3 step and the MoE
+    # block beside it.
+    by_name = {r["op"]: r for r in op_rows}
+    roofline_mfma = None
+    lg = by_name.get("c3.logits gemm [1024,4096]x[4096,128256]")
+    if lg is not None:
+        roofline_mfma = {"kernel": "gemm_kernel<bf16, bf16, 256x256x64, 8 waves, A K-contiguous, B K-contiguous> (LM-head logits, "
+                                   "one 1024-token chunk)",
+                         "bound": "mfma", "achieved": lg["achieved"], "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": lg["frac"], "flop_per_launch": lg["algorithmic"], "avg_ms": lg["ms"]}
+        for key, prefix in (("c3_step_reference_schedule", "c3.lm_head fwd+bwd (chunk 1024, one GEMM group per chunk and bf16"),
+                            ("c3_step_8_chunks_per_group_opt_in", "c3.lm_head fwd+bwd (chunk 1024 x 8"),
+                            ("c5_moe_block", "c5.moe block fwd+bwd")):
+            row = next((r for r in op_rows if r["op"].startswith(prefix)), None)
+            if row is not None:
+                roofline_mfma[key] = {"ms": row["ms"], "achieved": row["achieved"], "frac": row["frac"]}
+
+    # Last key of the line on purpose: a reader who keeps only the end of the output still sees one
+    # figure per configuration (milliseconds, fraction of the roofline that bounds the row).
+    def brief(prefix, label):
+        row = next((r for r in op_rows if r["op"].startswith(prefix)), None)
+        return None if row is None else f"{label} {row['ms']}ms {row['frac']}"
+
+    summary = [t for t in (
+        brief("c1.rmsnorm_fwd", "c1.norm_fwd"), brief("c1.rmsnorm_bwd(dX+=,dW+=)", "c1.norm_bwd"),
+        brief("c1x16.rmsnorm_fwd", "c1x16.norm_fwd"), brief("c1x16.rmsnorm_bwd", "c1x16.norm_bwd"),
+        brief("c2.rope_fwd", "c2.rope_fwd"), brief("c2.rope_bwd", "c2.rope_bwd"), brief("c2.swiglu_fwd", "c2.swiglu_fwd"),
+        brief("c2.swiglu_bwd", "c2.swiglu_bwd"),
+        brief("c3.lm_head fwd+bwd (chunk 1024, one GEMM group per chunk and bf16", "c3.head chunk1024 bf16dW(ref schedule)"),
+        brief("c3.lm_head fwd+bwd (chunk 1024, one GEMM group per chunk, fp32", "c3.head chunk1024 fp32dW"),
+        brief("c3.lm_head fwd+bwd (chunk 1024 x 8", "c3.head 8chunks(opt-in) fp32dW"),
+        brief("c3.logits gemm [", "c3.logits"), brief("c3.dW gemm [128256,1024]x[1024,4096] (+= fp32)", "c3.dW fp32"),
+        brief("c3.dW gemm [128256,1024]x[1024,4096] (+= bf16)", "c3.dW bf16"), brief("c3.dX gemm [", "c3.dX"),
+        brief("c3.softmax_ce", "c3.softmax_ce"),
+        brief("c4.adamw(fp32 p/m/v, bf16 g, bf16 copy-out)", "c4.adamw+copy"), brief("c4.adamw(fp32 p/m/v, bf16 g)", "c4.adamw"),
+        brief("c5.moe block fwd (", "c5.moe_fwd"), brief("c5.moe block bwd", "c5.moe_bwd"), brief("c5.moe block fwd+bwd", "c5.moe"),
+        brief("moe_ref.routed MLP, the reference's micro-benchmark shape (16384 tokens, d 2048, F 512, 256 experts, top-8) fwd+bwd", "moe_ref"),
+        brief("ffn.gate gemm [", "ffn.gate"), brief("ffn.gate gemm, vendor", "ffn.gate vendor"),
+        brief("ffn.down gemm [", "ffn.down"), brief("ffn.down gemm, vendor", "ffn.down vendor"),
+        brief("ffn.dense block fwd+bwd", "ffn.block"), brief("attn.projections fwd+bwd", "attn.proj"),
+        brief("probe.save-level", "gemm8192^3")) if t is not None]
+
     result = {
         "metric": METRIC,
         "value": round(value, 1),
@@ -1006,8 +1150,10 @@ def main():
                    "algorithmic_bytes_per_step": step_bytes},
         "roofline": roofline,
         "cpu_baseline": cpu,
+        "roofline_mfma": roofline_mfma,
         "mfma_probe": mfma_probe,
         "ops": op_rows,
+        "summary": summary,
     }
     print(json.dumps(result))
 

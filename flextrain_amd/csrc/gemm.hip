@@ -222,6 +222,11 @@ struct DispatchContext {
     std::unordered_map<ShapeKey, int, ShapeHash> exact;   // full problem -> tile config
     std::unordered_map<ShapeKey, int, ShapeHash> fuzzy;   // dims rounded up to round_multiple
     uint64_t algos_saved = 0, calls = 0, hits = 0, total_ns = 0, hash_ns = 0, lookup_ns = 0, driver_ns = 0;
+    // the problem of the previous call and its configuration: a training loop repeats a handful of
+    // shapes back to back, and comparing 56 bytes is cheaper than hashing them
+    ShapeKey last_key{};
+    int last_cfg = 0;
+    bool has_last = false;
 };
 
 static inline uint64_t now_ns() {
@@ -278,8 +283,11 @@ extern "C" int dispatch_matmul(DispatchContext* ctx, intptr_t stream_ptr, int M,
     ShapeKey key{M, N, K, lda, ldb, ldc, ldd, a_dt, b_dt, c_dt, d_dt, trans_a, trans_b, key_facts(A, B, has_c)};
     const uint64_t h1 = now_ns();
     int cfg;
-    auto it = ctx->exact.find(key);
-    if (it != ctx->exact.end()) {
+    std::unordered_map<ShapeKey, int, ShapeHash>::iterator it;
+    if (ctx->has_last && ctx->last_key == key) {
+        cfg = ctx->last_cfg;
+        ctx->hits++;
+    } else if ((it = ctx->exact.find(key)) != ctx->exact.end()) {
         cfg = it->second;
         ctx->hits++;
     } else {
@@ -303,6 +311,9 @@ extern "C" int dispatch_matmul(DispatchContext* ctx, intptr_t stream_ptr, int M,
         }
         ctx->exact[key] = cfg;
     }
+    ctx->last_key = key;
+    ctx->last_cfg = cfg;
+    ctx->has_last = true;
     if ((cfg >> 8) > 1 && (!part || (size_t)(cfg >> 8) * M * N * sizeof(float) > workspace_bytes))
         cfg &= 0xff;  // cached with K splits, but this call lends no (or too small a) workspace
     const uint64_t h2 = now_ns();

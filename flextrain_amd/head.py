@@ -29,14 +29,15 @@ class LMHeadConfig:
     vocab_size: int
     rms_norm_eps: float = 1e-5
     head_chunk_size: int = 1024
-    # Micro-chunks handled by one GEMM group (not in the reference, which holds one logits buffer of
-    # head_chunk_size rows).  None: as many as keep the logits buffer under ``logits_buffer_bytes``;
-    # the default bound, 512 MiB, admits two 1024-token chunks at a 128256-entry vocabulary (525 MB
-    # against the reference's 263 MB), 1 selects the reference's schedule exactly.  Larger groups mean
-    # fewer read-modify-write passes over the head weight gradient and better-filled GEMMs (8 chunks,
-    # a 2.1 GB buffer, are a fifth faster than 1); the result differs only in accumulation order.
-    fuse_chunks: int | None = None
-    logits_buffer_bytes: int = 512 << 20
+    # Micro-chunks handled by one GEMM group.  1 (default) is the reference's schedule: one logits
+    # buffer of head_chunk_size rows (263 MB at a 128256-entry vocabulary).  Larger groups are an
+    # opt-in trade of memory for time (not in the reference): fewer read-modify-write passes over the
+    # head weight gradient and better-filled GEMMs; the result differs only in accumulation order.
+    # Measured at 8192 tokens x 128256: 2 chunks (525 MB) are no faster than 1, because the buffer no
+    # longer fits the 256 MB last-level cache between the GEMMs and the loss kernel; 8 chunks (2.1 GB)
+    # are a fifth faster.  None: as many chunks as keep the buffer under ``logits_buffer_bytes``.
+    fuse_chunks: int | None = 1
+    logits_buffer_bytes: int = 4 << 30
     final_logit_softcap: float | None = None
     compute_dtype: torch.dtype = torch.bfloat16
     master_dtype: torch.dtype | None = None

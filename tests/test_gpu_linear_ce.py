@@ -279,9 +279,9 @@ def test_lm_head_skips_missing_grads_and_bf16_accumulator(dev):
 def test_full_size_llama_head(dev):
     """hidden [8192,4096], lm_head [128256,4096], 10 % ignored labels, micro-chunk 1024.  The oracle runs
     on a sample of token rows (whole vocabulary rows of logits, loss, dZ and the row's dx); everything
-    else is checked through properties that hold at any size: the default schedule (two chunks per GEMM
-    group), the 8-chunk groups and the per-chunk schedule agree, ignored rows have zero loss, and the head
-    gradient sums to ~0 over the vocabulary (every kept row of dZ sums to 0)."""
+    else is checked through properties that hold at any size: two-chunk groups, eight-chunk groups and the
+    per-chunk schedule (the default) agree, ignored rows have zero loss, and the head gradient sums to ~0
+    over the vocabulary (every kept row of dZ sums to 0)."""
     T, d, V, chunk = 8192, 4096, 128256, 1024
     g = gen(1002)
     x = randn(g, T, d)
@@ -302,7 +302,7 @@ def test_full_size_llama_head(dev):
                                           loss_fn=loss_fn)
         return dx, stats, gh, gn
 
-    dx, stats, gh, gn = run(None)
+    dx, stats, gh, gn = run(2)
     dx8, stats8, gh8, gn8 = run(8)
     keep = _KeepLogits(CrossEntropyLoss())
     dx1, stats1, gh1, gn1 = run(1, keep)
@@ -331,7 +331,7 @@ def test_full_size_llama_head(dev):
     keep.kept.clear()
     del wf
     close(stats8.per_token_loss, stats1.per_token_loss, rtol=1e-4, atol=1e-4, what="loss, 8-chunk groups vs per chunk")
-    for what, got_h, got_n, got_x in (("per chunk", gh1, gn1, dx1), ("default groups", gh, gn, dx), ("8-chunk groups", gh8, gn8, dx8)):
+    for what, got_h, got_n, got_x in (("per chunk", gh1, gn1, dx1), ("2-chunk groups", gh, gn, dx), ("8-chunk groups", gh8, gn8, dx8)):
         close(got_h.cpu()[vs], gh_ref, rtol=1e-2, atol=1e-2 * gh_ref.abs().max().item(), what=f"g_head rows, {what}")
         close(got_n, gn_ref, rtol=1e-2, atol=1e-2 * gn_ref.abs().max().item(), what=f"g_norm, {what}")
         close(got_x, dx_all, rtol=1e-2, atol=1e-2 * dx_all.float().abs().max().item(), what=f"dx of all tokens, {what}")
