@@ -85,14 +85,14 @@ _SIGNATURES = {
     "fx_grouped_gemm_rows_swiglu_bwd": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int, c_void_p, c_int64,
                                                 c_void_p, c_int, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int,
                                                 c_void_p, c_int, c_int64, c_int, c_int, c_int, c_void_p, c_size_t,
-                                                c_void_p, c_size_t, c_void_p]),
+                                                c_void_p, c_size_t, c_void_p, c_int64, c_void_p]),
     "fx_grouped_ws_bytes": (c_size_t, [c_int, c_int64]),
     "fx_grouped_gemm_rows": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int, c_void_p, c_int64,
                                      c_void_p, c_int64, c_void_p, c_int, c_int64, c_int, c_int, c_float, c_float,
                                      c_int, c_void_p, c_size_t, c_void_p]),
     "fx_grouped_gemm_wgrad": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int,
                                       c_void_p, c_int, c_int64, c_int, c_int, c_float, c_float, c_int, c_void_p,
-                                      c_size_t, c_void_p]),
+                                      c_size_t, c_void_p, c_int64, c_void_p, c_int64, c_void_p]),
     "fx_grouped_gemm_rows_glu": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int, c_int64, c_void_p,
                                          c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int, c_int64, c_int,
                                          c_int, c_int, c_int, c_void_p, c_size_t, c_void_p, c_int64, c_void_p]),

@@ -49,6 +49,11 @@ struct OperandView {
     // row_map[origin + r] of `base` instead of row origin + r.
     const int32_t* row_map = nullptr;
     int map_rows = 0;          // rows of `base` a gathered tile may address: map entries are clamped to [0, map_rows)
+    // Gathered k-rows (M/N-contiguous tiles of the loaders that say so): k-row k of the operand is row
+    // k_map[k] of `base` instead of row k, for k in [0, k_ext).  The expert weight gradients read the
+    // unsorted activations that way: their contraction runs over an expert's rows.
+    const int32_t* k_map = nullptr;
+    int k_ext = 0;
     // tile row -> which matrix, and the index offset from `origin`
     __device__ __forceinline__ bool dual_second(int r) const { return (r & half) != 0; }
     __device__ __forceinline__ int dual_index(int r) const { return ((r & ~(2 * half - 1)) >> 1) + (r & (half - 1)); }

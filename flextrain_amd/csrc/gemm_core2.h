@@ -81,7 +81,12 @@ FX_DEV void stage2_load(Staged2<ROWS, NT>& st, const OperandView<T>& op, int k0,
 #pragma unroll
         for (int j = 0; j < N; ++j) {
             const int k = k0 + kb * 8 + part * N + j;
-            st.v[j] = k < K ? ldg16(op.base + (int64_t)k * op.ld + g) : zero;
+            if (k < K) {
+                const int64_t row = op.k_map != nullptr ? (int64_t)min(max(op.k_map[k], 0), op.map_rows - 1) : (int64_t)k;
+                st.v[j] = ldg16(op.base + row * op.ld + g);
+            } else {
+                st.v[j] = zero;
+            }
         }
     }
 }
@@ -380,6 +385,63 @@ struct TileLoaderV {
     }
 };
 
+// M/N-contiguous tile whose k-rows are gathered through OperandView::k_map.  A lane's column offset
+// is fixed; its rows change with every K-step, so the byte offsets are rebuilt per step from map
+// entries that were requested one step earlier:
+//   fetch()    request the map entries of the step after the one about to be issued (clamped to the
+//              mapped range, so it may always be called)
+//   prepare()  turn the entries on hand into byte offsets; called once per step before its first
+//              issue, i.e. right after the K loop's barrier, when no tile load is in flight (the
+//              compiler's wait for the entries then costs nothing)
+// The whole source must stay below 4 GB (32-bit lane offsets from the operand's base).
+template <typename T, int ROWS, int NW>
+struct TileLoaderKG {
+    static constexpr int NI = ROWS / 8 / NW;
+    static constexpr int CPR = ROWS / 8, KPI = 64 / CPR;
+    static_assert(ROWS % (8 * NW) == 0 && (ROWS == 64 || ROWS == 128 || ROWS == 256), "see TileLoader");
+    unsigned col[NI], roff[NI];
+    int nidx[NI];
+    const T* base;
+    const int32_t* kmap;
+    int kpos, kext, map_rows;
+    unsigned ld_bytes;
+
+    FX_DEV void fetch() {
+#pragma unroll
+        for (int j = 0; j < NI; ++j) {
+            const int kk = min(kpos + j * NW * KPI, kext - 1);
+            nidx[j] = kmap[kk < 0 ? 0 : kk];
+        }
+        kpos += GEMM_BK;
+    }
+    FX_DEV void prepare() {
+#pragma unroll
+        for (int j = 0; j < NI; ++j) roff[j] = col[j] + (unsigned)min(max(nidx[j], 0), map_rows - 1) * ld_bytes;
+    }
+    FX_DEV void init(const OperandView<T>& op, int wave, int lane) {
+        const int kin = lane / CPR, pos = lane % CPR;
+#pragma unroll
+        for (int j = 0; j < NI; ++j) {
+            const int k = (j * NW + wave) * KPI + kin;
+            const int c = pos ^ (swz_tr(k) % CPR);
+            int g = op.origin + c * 8;
+            g = g + 8 <= op.ext ? g : op.ext - 8;
+            col[j] = (unsigned)((g - op.origin) * (int)sizeof(T));
+        }
+        base = op.base + op.origin;
+        kmap = op.k_map;
+        kext = op.k_ext;
+        map_rows = op.map_rows;
+        ld_bytes = (unsigned)(op.ld * (int64_t)sizeof(T));
+        kpos = wave * KPI + kin;
+        fetch();
+    }
+    template <int J>
+    FX_DEV void issue(T* lds, int wave) {
+        load_to_lds16_s(roff[J], base, (unsigned)(uintptr_t)(lds + (J * NW + wave) * 512));
+    }
+};
+
 // Epilogue.  The accumulators hold the transposed tile (MFMA is called with the B fragment
 // first): lane l, register v of acc[i][j] is D[row0 + 32i + l%32][col0 + 32j + 8*(v/4) + 4*(l/32) + v%4],
 // i.e. a lane owns groups of 4 consecutive columns.  Each wave stages one 32-row band at a time in
@@ -497,16 +559,20 @@ constexpr size_t gemm2_lds_bytes() {
 // Between the two the caller may do anything that leaves buf0 alone and issues no inline-assembly
 // loads of its own (compiler-generated loads and stores are fine: the counted waits below only
 // assume that loads complete in the order they were issued).
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_MN, bool B_MN, bool B_DUAL = false, bool ZERO = true>
+// A_KG / B_KG: that operand (M/N-contiguous) gathers its k-rows through OperandView::k_map.
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_MN, bool B_MN, bool B_DUAL = false, bool ZERO = true,
+          bool A_KG = false, bool B_KG = false>
 struct MainLoop2 {
     static constexpr int NW = WAVES_M * WAVES_N, NT = NW * 64;
     static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     static constexpr int TM = WM / 32, TN = WN / 32;
     static constexpr int BUF = (BM + BN) * GEMM_BK;
     typedef MmaPipe<T, BM, BN, WM, WN, A_MN, B_MN> Pipe;
-    typedef TileLoader<T, BM, NW, A_MN, false> LoadA;
+    static_assert((!A_KG || A_MN) && (!B_KG || (B_MN && !B_DUAL)), "only M/N-contiguous single-matrix tiles gather k-rows");
+    typedef typename std::conditional<A_KG, TileLoaderKG<T, BM, NW>, TileLoader<T, BM, NW, A_MN, false>>::type LoadA;
     typedef typename std::conditional<(B_MN && B_DUAL), TileLoaderV<T, BN, NW, B_MN, B_DUAL>,
-                                      TileLoader<T, BN, NW, B_MN, B_DUAL>>::type LoadB;
+                                      typename std::conditional<B_KG, TileLoaderKG<T, BN, NW>,
+                                                                TileLoader<T, BN, NW, B_MN, B_DUAL>>::type>::type LoadB;
     static constexpr int LD = LoadA::NI + LoadB::NI;            // load instructions per wave and K-step
     static constexpr int PER = (LD + Pipe::MFMAS - 1) / Pipe::MFMAS;
     static_assert(GEMM_BK == 64, "the pipeline below is written out for four sub-steps per K-step");
@@ -518,8 +584,16 @@ struct MainLoop2 {
     // instruction IDX of the next K-step into the stage at `buf` (K-steps are issued in order)
     template <int IDX>
     FX_DEV void issue_one(T* buf) {
+        if constexpr (IDX == 0) {           // a new step: gathered operands turn their map entries into offsets
+            if constexpr (A_KG) la.prepare();
+            if constexpr (B_KG) lb.prepare();
+        }
         if constexpr (IDX < LoadA::NI) la.template issue<IDX>(buf, wave);
         else if constexpr (IDX < LD) lb.template issue<IDX - LoadA::NI>(buf + BM * GEMM_BK, wave);
+        if constexpr (IDX == LD - 1) {      // the step is out: request the entries of the one after
+            if constexpr (A_KG) la.fetch();
+            if constexpr (B_KG) lb.fetch();
+        }
     }
     FX_DEV void issue(T* buf) { static_for<0, LD>([&](auto idx) { issue_one<decltype(idx)::value>(buf); }); }
 

@@ -332,7 +332,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void grouped_rows_swiglu_bw
     const T* __restrict__ XUP, int64_t ldx, const TW* __restrict__ SRW, T* __restrict__ DXUP, int64_t lddx,
     T* __restrict__ ACT, int64_t ldact, float* __restrict__ PART, const int32_t* __restrict__ NTILES,
     const int32_t* __restrict__ OFFSETS, const int32_t* __restrict__ TILES, int F, int K, int tiles_n, int E,
-    int max_tiles) {
+    int max_tiles, const int32_t* __restrict__ A_ROW_MAP, int a_rows) {
     static_assert((BM + BN) * GEMM_BK * sizeof(T) == 64 * 1024, "the LDS plan assumes 64 KB stages");
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T* smem = reinterpret_cast<T*>(smem_raw);
@@ -353,7 +353,12 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void grouped_rows_swiglu_bw
         t.rows = OFFSETS[t.e + 1] - OFFSETS[t.e];
         return t;
     };
-    auto view_a = [&](const Tile& t) { return OperandView<T>{A + t.row0 * lda, lda, t.rows, t.m0}; };
+    // A_ROW_MAP: expert-sorted row r is row A_ROW_MAP[r] of the unsorted A (gathered by the tile loads)
+    auto view_a = [&](const Tile& t) {
+        OperandView<T> v{A_ROW_MAP ? A : A + t.row0 * lda, lda, t.rows, t.m0};
+        if (A_ROW_MAP) { v.row_map = A_ROW_MAP + t.row0; v.map_rows = a_rows; }
+        return v;
+    };
     auto view_b = [&](const Tile& t) { return OperandView<T>{B + (int64_t)t.e * b_expert_stride, ldb, F, t.tn * BN}; };
     MainLoop2<T, BM, BN, WAVES_M, WAVES_N, false, B_MN> loop;
     Tile cur = lookup(pid);
@@ -396,11 +401,14 @@ __global__ __launch_bounds__(256) void dprob_reduce_kernel(const float* __restri
     DW[r] = (TDW)s;
 }
 
-template <typename T, typename TG, int BM, int BN, int WAVES_M, int WAVES_N>
+// KG: 0 = A and B are expert-sorted; 1 = A, 2 = B is the UNSORTED (src_rows, *) matrix and sorted row r
+// of it is row KMAP[r] (the expert-sorted copy of that operand is then never made).
+template <typename T, typename TG, int BM, int BN, int WAVES_M, int WAVES_N, int KG>
 __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void grouped_wgrad_walk_kernel(
     const T* __restrict__ A, int64_t lda, const T* __restrict__ B, int64_t ldb, TG* G, int64_t ldg,
     int64_t g_expert_stride, const int32_t* __restrict__ NTILES, const int32_t* __restrict__ OFFSETS, int M, int N,
-    float alpha, float beta, int tiles_n, int tiles_per_expert, int total, int E) {
+    float alpha, float beta, int tiles_n, int tiles_per_expert, int total, int E, const int32_t* __restrict__ KMAP,
+    int src_rows) {
     static_assert((BM + BN) * GEMM_BK * sizeof(T) == 64 * 1024, "the LDS plan assumes 64 KB stages");
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T* smem = reinterpret_cast<T*>(smem_raw);
@@ -420,9 +428,17 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void grouped_wgrad_walk_ker
         t.rows = OFFSETS[t.e + 1] - OFFSETS[t.e];
         return t;
     };
-    auto view_a = [&](const Tile& t) { return OperandView<T>{A + t.row0 * lda, lda, M, t.tm * BM}; };
-    auto view_b = [&](const Tile& t) { return OperandView<T>{B + t.row0 * ldb, ldb, N, t.tn * BN}; };
-    MainLoop2<T, BM, BN, WAVES_M, WAVES_N, true, true> loop;
+    auto view_a = [&](const Tile& t) {
+        OperandView<T> v{KG == 1 ? A : A + t.row0 * lda, lda, M, t.tm * BM};
+        if (KG == 1) { v.k_map = KMAP + t.row0; v.k_ext = t.rows; v.map_rows = src_rows; }
+        return v;
+    };
+    auto view_b = [&](const Tile& t) {
+        OperandView<T> v{KG == 2 ? B : B + t.row0 * ldb, ldb, N, t.tn * BN};
+        if (KG == 2) { v.k_map = KMAP + t.row0; v.k_ext = t.rows; v.map_rows = src_rows; }
+        return v;
+    };
+    MainLoop2<T, BM, BN, WAVES_M, WAVES_N, true, true, false, true, KG == 1, KG == 2> loop;
     Tile cur = lookup(pid);
     OperandView<T> a = view_a(cur), b = view_b(cur);
     loop.begin(a, b, cur.rows, WalkLds<T>::buf0(smem));
@@ -618,7 +634,8 @@ extern "C" int fx_grouped_gemm_rows_glu(const void* A, int64_t lda, const void* 
 extern "C" int fx_grouped_gemm_wgrad(const void* A, int64_t lda, const void* B, int64_t ldb, void* G, int64_t ldg,
                                      int64_t g_expert_stride, int g_dt, const int32_t* counts, int E,
                                      int64_t total_rows, int M, int N, float alpha, float beta, int dt, void* ws,
-                                     size_t ws_bytes, hipStream_t stream) {
+                                     size_t ws_bytes, const int32_t* a_row_map, int64_t a_rows,
+                                     const int32_t* b_row_map, int64_t b_rows, hipStream_t stream) {
     if (E <= 0 || total_rows < 0 || M <= 0 || N <= 0) FX_FAIL("fx_grouped_gemm_wgrad: bad shape");
     if (!A || !B || !G) FX_FAIL("fx_grouped_gemm_wgrad: null pointer");
     if (!ws || ws_bytes < fx_grouped_ws_bytes(E, total_rows)) FX_FAIL("fx_grouped_gemm_wgrad: workspace too small");
@@ -627,6 +644,12 @@ extern "C" int fx_grouped_gemm_wgrad(const void* A, int64_t lda, const void* B, 
     if (g_dt != dt && !(dt == DT_BF16 && g_dt == DT_F32)) FX_FAIL("fx_grouped_gemm_wgrad: G must match the inputs or be fp32 (bf16 inputs)");
     if (!aligned16(A) || !aligned16(B) || (lda & 7) || (ldb & 7) || (M & 7) || (N & 7))
         FX_FAIL("fx_grouped_gemm_wgrad: operands must be 16-byte aligned with M and N multiples of 8");
+    if (a_row_map && b_row_map) FX_FAIL("fx_grouped_gemm_wgrad: at most one operand may be gathered through a row map");
+    if (a_row_map && (a_rows <= 0 || a_rows > 0x7fffffff || (uint64_t)a_rows * (uint64_t)lda * 2u >= (1ull << 32)))
+        FX_FAIL("fx_grouped_gemm_wgrad: a gathered A must have a_rows > 0 and stay below 4 GB");
+    if (b_row_map && (b_rows <= 0 || b_rows > 0x7fffffff || (uint64_t)b_rows * (uint64_t)ldb * 2u >= (1ull << 32)))
+        FX_FAIL("fx_grouped_gemm_wgrad: a gathered B must have b_rows > 0 and stay below 4 GB");
+    if (total_rows == 0 && (a_row_map || b_row_map)) { a_row_map = nullptr; b_row_map = nullptr; }
     GroupedWs w = split_ws(ws, E);
     if (counts) {    // only the row offsets are used here; the plan is the one every entry point writes for this shape
         grouped_plan_kernel<<<1, 256, 0, stream>>>(counts, E, rows_bm(total_rows, E), w.ntiles, w.offsets, w.tiles);
@@ -635,20 +658,29 @@ extern "C" int fx_grouped_gemm_wgrad(const void* A, int64_t lda, const void* B, 
     constexpr int BM = 256, BN = 256;
     const int tiles_m = cdiv_i(M, BM), tiles_n = cdiv_i(N, BN);
     const dim3 grid((unsigned)(tiles_m * tiles_n) * (unsigned)E);
-#define FX_WG_WALK(TT, TG)                                                                                \
+    const unsigned grid_w = grid.x < (unsigned)walk_grid() ? grid.x : (unsigned)walk_grid();
+    const int32_t* kmap = a_row_map ? a_row_map : b_row_map;
+    const int src_rows = (int)(a_row_map ? a_rows : (b_row_map ? b_rows : 0));
+#define FX_WG_LAUNCH(TT, TG, KG_)                                                                         \
     {                                                                                                     \
-        auto kern = grouped_wgrad_walk_kernel<TT, TG, BM, BN, 2, 4>;                                      \
+        auto kern = grouped_wgrad_walk_kernel<TT, TG, BM, BN, 2, 4, KG_>;                                 \
         FX_ENSURE_DYNAMIC_LDS(kern, kWalkLdsBytes);                                                       \
-        const unsigned grid_w = grid.x < (unsigned)walk_grid() ? grid.x : (unsigned)walk_grid();          \
         kern<<<dim3(grid_w), 2 * 4 * 64, kWalkLdsBytes, stream>>>(                                        \
             reinterpret_cast<const TT*>(A), lda, reinterpret_cast<const TT*>(B), ldb, reinterpret_cast<TG*>(G), ldg, \
             g_expert_stride, w.ntiles, w.offsets, M, N, alpha, beta, tiles_n, tiles_m * tiles_n,          \
-            (int)grid.x, E);                                                                              \
+            (int)grid.x, E, kmap, src_rows);                                                              \
+    }
+#define FX_WG_WALK(TT, TG)                                                                                \
+    {                                                                                                     \
+        if (a_row_map) FX_WG_LAUNCH(TT, TG, 1)                                                            \
+        else if (b_row_map) FX_WG_LAUNCH(TT, TG, 2)                                                       \
+        else FX_WG_LAUNCH(TT, TG, 0)                                                                      \
     }
     if (dt == DT_BF16 && g_dt == DT_BF16) FX_WG_WALK(bf16, bf16)
     else if (dt == DT_BF16) FX_WG_WALK(bf16, float)
     else FX_WG_WALK(f16, f16)
 #undef FX_WG_WALK
+#undef FX_WG_LAUNCH
     FX_CHECK_LAUNCH("fx_grouped_gemm_wgrad");
     return 0;
 }
@@ -665,7 +697,8 @@ extern "C" int fx_grouped_gemm_rows_swiglu_bwd(const void* dy, int64_t lddy, con
                                                const void* srw, int srw_dt, void* dx_up, int64_t lddx, void* fwd_act,
                                                int64_t ldact, void* dprob, int dprob_dt, const int32_t* counts, int E,
                                                int64_t total_rows, int F, int K, int dt, void* ws, size_t ws_bytes,
-                                               void* part_ws, size_t part_ws_bytes, hipStream_t stream) {
+                                               void* part_ws, size_t part_ws_bytes, const int32_t* dy_row_map,
+                                               int64_t dy_rows, hipStream_t stream) {
     if (E <= 0 || total_rows < 0 || F <= 0 || K <= 0) FX_FAIL("fx_grouped_gemm_rows_swiglu_bwd: bad shape");
     if (total_rows == 0) return 0;
     if (!dy || !w_down || !x_up || !srw || !dx_up || !dprob) FX_FAIL("fx_grouped_gemm_rows_swiglu_bwd: null pointer");
@@ -681,6 +714,8 @@ extern "C" int fx_grouped_gemm_rows_swiglu_bwd(const void* dy, int64_t lddy, con
         (lddy & 7) || (ldb & 7) || (ldx & 7) || (lddx & 7) || (fwd_act && (ldact & 7)) || (K & 7) || (F & 7) ||
         (b_expert_stride & 7))
         FX_FAIL("fx_grouped_gemm_rows_swiglu_bwd: operands must be 16-byte aligned with K, F and every row stride a multiple of 8");
+    if (dy_row_map && (dy_rows <= 0 || dy_rows > 0x7fffffff || (uint64_t)dy_rows * (uint64_t)lddy * 2u >= (1ull << 32)))
+        FX_FAIL("fx_grouped_gemm_rows_swiglu_bwd: a gathered dy must have dy_rows > 0 and stay below 4 GB");
     if (ldx < 2 * (int64_t)F || lddx < 2 * (int64_t)F || (fwd_act && ldact < F)) FX_FAIL("fx_grouped_gemm_rows_swiglu_bwd: x_up / dx_up rows hold 2 F elements, fwd_act rows F");
     GroupedWs w = split_ws(ws, E);
     constexpr int BM = 256;
@@ -700,7 +735,7 @@ extern "C" int fx_grouped_gemm_rows_swiglu_bwd(const void* dy, int64_t lddy, con
             reinterpret_cast<const TT*>(dy), lddy, reinterpret_cast<const TT*>(w_down), ldb, b_expert_stride, \
             reinterpret_cast<const TT*>(x_up), ldx, reinterpret_cast<const TW*>(srw), reinterpret_cast<TT*>(dx_up), \
             lddx, reinterpret_cast<TT*>(fwd_act), ldact, reinterpret_cast<float*>(part_ws), w.ntiles, w.offsets, \
-            w.tiles, F, K, tiles_n, E, (int)max_tiles);                                                   \
+            w.tiles, F, K, tiles_n, E, (int)max_tiles, dy_row_map, (int)dy_rows);                         \
     }
 #define FX_SWB_T(TT)                                                                                      \
     if (srw_dt == DT_F32) { if (trans_b) FX_SWB(TT, float, false) else FX_SWB(TT, float, true) }          \

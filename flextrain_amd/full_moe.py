@@ -22,6 +22,7 @@ from .ops.grouped import (
     flextrain_grouped_gemm_rows_glu,
     flextrain_grouped_gemm_rows_swiglu_bwd,
     flextrain_grouped_gemm_wgrad,
+    gathered_operand_supported,
     grouped_glu_supported,
     grouped_swiglu_bwd_supported,
 )
@@ -140,36 +141,61 @@ def swiglu_expert_loop_fwd(scattered_x, x_preact_buf, w_up, w_down, expert_count
         flextrain_grouped_gemm_rows(act, w_down.transpose(1, 2), counts, scattered_x, plan=plan)
 
 
+def gathered_backward_supported(dy, x, w_down, x_preact_buf, srw, dx_up_up_grouped, dprobs):
+    """Whether the expert backward can read the token rows of ``dy`` and ``x`` in place through a row
+    map (the fused dgrad launch and the gathering weight-gradient launches must take the operands).
+    ``x_preact_buf``, ``srw``, ``dx_up_up_grouped`` and ``dprobs`` hold exactly the routed rows."""
+    return (gathered_operand_supported(dy) and gathered_operand_supported(x) and dy.shape == x.shape
+            and grouped_swiglu_bwd_supported(dy, w_down, x_preact_buf, srw, dx_up_up_grouped, None, dprobs,
+                                             dy_is_unsorted=True))
+
+
 def swiglu_expert_loop_bwd(scattered_upstream, scattered_x, x_preact_buf, srw, dprobs, w_up, w_down, grads,
                            expert_counts_cpu, dx_up_up_grouped, dx_pre_grouped, *, expert_dim, primary_stream,
-                           secondary_stream=None, expert_counts_gpu=None):
+                           secondary_stream=None, expert_counts_gpu=None, gather_dy=None, gather_x=None,
+                           row_sources=None):
     """Backward of the expert block on expert-sorted rows (steps a-e of
     flextrain/ops/full_moe.py:499-626): dgrad through ``w_down``, SwiGLU backward
     (per-row router-weight gradient into ``dprobs``), ``g_down[e] +=``, dgrad
     through ``w_up`` into ``dx_pre_grouped``, ``g_up[e] +=``.  A gradient
-    accumulator missing from ``grads`` (or None) is skipped."""
-    TK = scattered_upstream.shape[0]
+    accumulator missing from ``grads`` (or None) is skipped.
+
+    ``gather_dy`` / ``gather_x`` / ``row_sources`` (not in the reference): the unsorted ``(T, d)``
+    upstream gradient and activations and the token of every expert-sorted row; the launches that read
+    ``dy`` and ``x`` then gather their rows from these, and ``scattered_upstream`` / ``scattered_x`` are
+    not read (they may be None): the backward makes no expert-sorted copy of either."""
+    TK = x_preact_buf.shape[0] if scattered_upstream is None else scattered_upstream.shape[0]
     counts = _device_counts(expert_counts_cpu, expert_counts_gpu)
+    gathered = gather_dy is not None
+    if gathered and (gather_x is None or row_sources is None):
+        raise ValueError("gather_dy, gather_x and row_sources go together")
+    dy_src = gather_dy if gathered else scattered_upstream
     # One stream: every grouped launch fills all CUs with one resident workgroup each, so launches on a
     # second stream only take CUs from the first (measured at 8192 tokens x 128 experts: weight
     # gradients on the secondary stream 2.06 ms against 2.01 ms for the same work on one stream).
     with torch.cuda.stream(primary_stream):
-        fwd_act = torch.empty((TK, expert_dim), dtype=scattered_upstream.dtype, device=scattered_upstream.device)
-        plan = GroupedPlan(counts, w_up.shape[0], TK, scattered_upstream.device)
+        fwd_act = torch.empty((TK, expert_dim), dtype=dy_src.dtype, device=dy_src.device)
+        plan = GroupedPlan(counts, w_up.shape[0], TK, dy_src.device)
         dx_up, x_up, rw, dpr = dx_up_up_grouped[:TK], x_preact_buf[:TK], srw[:TK], dprobs[:TK]
-        if grouped_swiglu_bwd_supported(scattered_upstream, w_down, x_up, rw, dx_up, fwd_act, dpr):
+        if gathered or grouped_swiglu_bwd_supported(dy_src, w_down, x_up, rw, dx_up, fwd_act, dpr):
             # (a) + (b) in one launch: dx_act lives only in the dgrad's epilogue
-            flextrain_grouped_gemm_rows_swiglu_bwd(scattered_upstream, w_down, counts, x_up, rw, dx_up, dpr,
-                                                   fwd_act=fwd_act, plan=plan)
+            flextrain_grouped_gemm_rows_swiglu_bwd(dy_src, w_down, counts, x_up, rw, dx_up, dpr, fwd_act=fwd_act,
+                                                   plan=plan, row_sources=row_sources if gathered else None)
         else:
             dx_act = torch.empty_like(fwd_act)
             flextrain_grouped_gemm_rows(scattered_upstream, w_down, counts, dx_act, plan=plan)         # (a)
             flextrain_swiglu_moe_bwd(dx_act, x_up, rw, dx=dx_up, dw=dpr, fwd_act=fwd_act)               # (b)
-        if grads.get("g_down") is not None:
-            flextrain_grouped_gemm_wgrad(scattered_upstream, fwd_act, grads["g_down"], counts, plan=plan)   # (c)
-        flextrain_grouped_gemm_rows(dx_up_up_grouped[:TK], w_up, counts, dx_pre_grouped[:TK], plan=plan)    # (d)
-        if grads.get("g_up") is not None:
-            flextrain_grouped_gemm_wgrad(dx_up_up_grouped[:TK], scattered_x, grads["g_up"], counts, plan=plan)  # (e)
+        if grads.get("g_down") is not None:                                                                 # (c)
+            if gathered:
+                flextrain_grouped_gemm_wgrad(gather_dy, fwd_act, grads["g_down"], counts, plan=plan, a_row_sources=row_sources)
+            else:
+                flextrain_grouped_gemm_wgrad(scattered_upstream, fwd_act, grads["g_down"], counts, plan=plan)
+        flextrain_grouped_gemm_rows(dx_up, w_up, counts, dx_pre_grouped[:TK], plan=plan)                    # (d)
+        if grads.get("g_up") is not None:                                                                   # (e)
+            if gathered:
+                flextrain_grouped_gemm_wgrad(dx_up, gather_x, grads["g_up"], counts, plan=plan, b_row_sources=row_sources)
+            else:
+                flextrain_grouped_gemm_wgrad(dx_up, scattered_x, grads["g_up"], counts, plan=plan)
 
 
 def swiglu_expert_loop_recompute_x_up(scattered_x, x_preact_buf, w_up, expert_counts_cpu, *, primary_stream,
@@ -251,4 +277,5 @@ __all__ = (
     "swiglu_expert_loop_bwd",
     "swiglu_expert_loop_recompute_x_up",
     "gathered_up_projection_supported",
+    "gathered_backward_supported",
 )

@@ -141,23 +141,35 @@ class FlextrainMoEExpertCompute:
         num_experts = weights["w_up"].shape[0]
         expert_dim = weights["w_down"].shape[2]
         host_counts = self._host_counts(chunk_extra, layer_id, num_experts)
-        scattered_upstream = scratch_fn((TK, d_model), dy.dtype)
-        flextrain_moe_scatter(dy, slot.index_mapping, out=scattered_upstream)
-        if recompute_handoff is not None:
-            scattered_x = recompute_handoff
-        else:
-            scattered_x = scratch_fn((TK, d_model), dy.dtype)
-            flextrain_moe_scatter(x, slot.index_mapping, out=scattered_x)
         srw = slot.scattered_router_weights[:TK, :]
         dprobs = torch.zeros_like(srw)
         dx_up_up_grouped = scratch_fn((TK, 2 * expert_dim), dy.dtype)
         dx_pre_grouped = scratch_fn((TK, d_model), dy.dtype)
+        # When the fused launches can take the operands they read the token rows of dy and x in place
+        # through the row map, and neither expert-sorted copy (one write and two reads of TK x d each) is
+        # made.  The LoRA capture hands the sorted copies on and a recompute hand-off already is one, so
+        # those two cases keep the scatter launches.
+        gathered = (lora_capture is None and recompute_handoff is None
+                    and full_moe.gathered_backward_supported(dy, x, weights["w_down"], slot.x_up[:TK], srw,
+                                                             dx_up_up_grouped, dprobs))
+        scattered_upstream = scattered_x = row_sources = None
+        if gathered:
+            row_sources = flextrain_moe_row_sources(slot.index_mapping, out=scratch_fn((TK,), torch.int32))
+        else:
+            scattered_upstream = scratch_fn((TK, d_model), dy.dtype)
+            flextrain_moe_scatter(dy, slot.index_mapping, out=scattered_upstream)
+            if recompute_handoff is not None:
+                scattered_x = recompute_handoff
+            else:
+                scattered_x = scratch_fn((TK, d_model), dy.dtype)
+                flextrain_moe_scatter(x, slot.index_mapping, out=scattered_x)
         full_moe.swiglu_expert_loop_bwd(
-            scattered_upstream=scattered_upstream, scattered_x=scattered_x, x_preact_buf=slot.x_up, srw=srw,
+            scattered_upstream=scattered_upstream, scattered_x=scattered_x, x_preact_buf=slot.x_up[:TK], srw=srw,
             dprobs=dprobs, w_up=weights["w_up"], w_down=weights["w_down"], grads=grads,
             expert_counts_cpu=host_counts, dx_up_up_grouped=dx_up_up_grouped, dx_pre_grouped=dx_pre_grouped,
             expert_dim=expert_dim, primary_stream=primary_stream, secondary_stream=secondary_stream,
-            expert_counts_gpu=slot.expert_counts)
+            expert_counts_gpu=slot.expert_counts, gather_dy=dy if gathered else None,
+            gather_x=x if gathered else None, row_sources=row_sources)
         if lora_capture is not None:
             lora_capture["scattered_x_grouped"] = scattered_x
             lora_capture["dx_up_up_grouped"] = dx_up_up_grouped

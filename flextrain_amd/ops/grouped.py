@@ -85,23 +85,51 @@ def flextrain_grouped_gemm_rows(A, B, counts, D, C=None, alpha=1.0, beta=0.0, pl
     return D
 
 
-def flextrain_grouped_gemm_wgrad(A, B, G, counts, alpha=1.0, beta=1.0, plan=None):
+def _row_sources_ok(row_sources, TK):
+    return (row_sources.dtype == torch.int32 and row_sources.numel() == TK and row_sources.is_contiguous()
+            and row_sources.is_cuda)
+
+
+def gathered_operand_supported(src):
+    """Whether an unsorted activation matrix can stand in for its expert-sorted copy in the grouped
+    launches that take ``row_sources`` (16-byte rows below 4 GB in all)."""
+    return (src.dim() == 2 and src.stride(1) == 1 and src.stride(0) % 8 == 0 and src.data_ptr() % 16 == 0
+            and src.dtype in (torch.bfloat16, torch.float16)
+            and src.shape[0] * src.stride(0) * src.element_size() < (1 << 32))
+
+
+def flextrain_grouped_gemm_wgrad(A, B, G, counts, alpha=1.0, beta=1.0, plan=None, a_row_sources=None,
+                                 b_row_sources=None):
     """``G[e] = alpha * A[rows_e].T @ B[rows_e] + beta * G[e]`` for every expert;
     ``A (TK, M)``, ``B (TK, N)`` expert-sorted, ``G (E, M, N)`` (bf16/fp16, or fp32
-    for bf16 inputs)."""
+    for bf16 inputs).
+
+    ``a_row_sources`` / ``b_row_sources`` (at most one; int32, one entry per expert-sorted row, from
+    ``flextrain_moe_row_sources``): that operand is then the UNSORTED ``(T, M)`` / ``(T, N)`` matrix and
+    sorted row ``r`` of it is row ``row_sources[r]``, gathered by the kernel's own tile loads."""
     _rowmajor(A, "A"), _rowmajor(B, "B")
     if G.dim() != 3 or G.stride(2) != 1:
         raise ValueError("G must be (E, M, N) with unit last stride")
     E, M, N = G.shape
-    TK = A.shape[0]
-    if A.shape[1] != M or B.shape[1] != N or B.shape[0] != TK:
+    if a_row_sources is not None and b_row_sources is not None:
+        raise ValueError("at most one operand may be gathered")
+    TK = B.shape[0] if a_row_sources is not None else A.shape[0]
+    for t, src, name in ((A, a_row_sources, "A"), (B, b_row_sources, "B")):
+        if src is None:
+            if t.shape[0] != TK:
+                raise ValueError(f"shape mismatch: A {tuple(A.shape)}, B {tuple(B.shape)}, G {tuple(G.shape)}")
+        elif not _row_sources_ok(src, TK) or not gathered_operand_supported(t):
+            raise ValueError(f"{name}: row sources must be a contiguous int32 CUDA tensor with {TK} elements and the "
+                             f"unsorted matrix must have 16-byte rows below 4 GB")
+    if A.shape[1] != M or B.shape[1] != N:
         raise ValueError(f"shape mismatch: A {tuple(A.shape)}, B {tuple(B.shape)}, G {tuple(G.shape)}")
     if A.dtype != B.dtype:
         raise TypeError("A and B must share a dtype")
     cptr, ws, nbytes = _plan_or_workspace(plan, counts, E, TK, A.device)
     rc = lib().fx_grouped_gemm_wgrad(ptr(A), A.stride(0), ptr(B), B.stride(0), ptr(G), G.stride(1), G.stride(0),
                                      dtype_enum(G.dtype), cptr, E, TK, M, N, alpha, beta,
-                                     dtype_enum(A.dtype), ptr(ws), nbytes, stream_ptr(A.device))
+                                     dtype_enum(A.dtype), ptr(ws), nbytes, ptr(a_row_sources), A.shape[0],
+                                     ptr(b_row_sources), B.shape[0], stream_ptr(A.device))
     check(rc, "fx_grouped_gemm_wgrad")
     return G
 
@@ -159,21 +187,26 @@ def flextrain_grouped_gemm_rows_glu(A, w_up, counts, pre, act, row_sources=None,
     return pre, act
 
 
-def grouped_swiglu_bwd_supported(dy, w_down, x_up, srw, dx_up, fwd_act, dprob):
+def grouped_swiglu_bwd_supported(dy, w_down, x_up, srw, dx_up, fwd_act, dprob, dy_is_unsorted=False):
     """Whether :func:`flextrain_grouped_gemm_rows_swiglu_bwd` can take these tensors (else the
-    caller runs the dgrad GEMM and ``flextrain_swiglu_moe_bwd`` separately)."""
+    caller runs the dgrad GEMM and ``flextrain_swiglu_moe_bwd`` separately).  ``dy_is_unsorted``:
+    ``dy`` is the ``(T, d)`` upstream gradient, to be gathered through row sources."""
     if dy.dtype not in (torch.bfloat16, torch.float16) or w_down.dim() != 3 or not w_down.is_contiguous():
         return False
     E, d, F = w_down.shape
-    TK = dy.shape[0]
+    TK = x_up.shape[0]
+    if dy_is_unsorted and not gathered_operand_supported(dy):
+        return False
     if any(t.dtype != dy.dtype for t in (w_down, x_up, dx_up)) or (fwd_act is not None and fwd_act.dtype != dy.dtype):
         return False
     if srw.dtype not in (dy.dtype, torch.float32) or dprob.dtype not in (dy.dtype, torch.float32):
         return False
     if not (srw.is_contiguous() and dprob.is_contiguous() and srw.numel() == TK and dprob.numel() == TK):
         return False
-    two_d = [dy, x_up, dx_up] + ([fwd_act] if fwd_act is not None else [])
+    two_d = [x_up, dx_up] + ([fwd_act] if fwd_act is not None else []) + ([] if dy_is_unsorted else [dy])
     if any(t.dim() != 2 or t.stride(1) != 1 or t.stride(0) % 8 or t.data_ptr() % 16 or t.shape[0] != TK for t in two_d):
+        return False
+    if dy.dim() != 2 or dy.stride(1) != 1 or dy.stride(0) % 8 or dy.data_ptr() % 16:
         return False
     if dy.shape[1] != d or x_up.shape[1] != 2 * F or dx_up.shape[1] != 2 * F or (fwd_act is not None and fwd_act.shape[1] != F):
         return False
@@ -181,17 +214,23 @@ def grouped_swiglu_bwd_supported(dy, w_down, x_up, srw, dx_up, fwd_act, dprob):
             and int(lib().fx_grouped_rows_tile_height(E, TK)) == 256)
 
 
-def flextrain_grouped_gemm_rows_swiglu_bwd(dy, w_down, counts, x_up, srw, dx_up, dprob, fwd_act=None, plan=None):
+def flextrain_grouped_gemm_rows_swiglu_bwd(dy, w_down, counts, x_up, srw, dx_up, dprob, fwd_act=None, plan=None,
+                                           row_sources=None):
     """Expert dgrad through ``w_down (E, d, F)`` with the weighted SwiGLU backward in its epilogue:
     ``dx_act = dy[rows_e] @ w_down[e]`` is rounded and consumed in registers;
     ``dx_up (TK, 2F)``, ``fwd_act (TK, F) = act * w`` and ``dprob (TK,) = sum_F dx_act * act`` are
     written.  ``x_up (TK, 2F)`` is the saved pre-activation ``[value | gate]``, ``srw`` the
     expert-sorted router weights.  ``dx_up`` / ``fwd_act`` equal, bit for bit, what
-    ``flextrain_grouped_gemm_rows`` + ``flextrain_swiglu_moe_bwd`` give."""
-    if not grouped_swiglu_bwd_supported(dy, w_down, x_up, srw, dx_up, fwd_act, dprob):
+    ``flextrain_grouped_gemm_rows`` + ``flextrain_swiglu_moe_bwd`` give.
+
+    ``row_sources``: ``dy`` is then the UNSORTED ``(T, d)`` upstream gradient and sorted row ``r`` is
+    ``dy[row_sources[r]]`` (no expert-sorted copy of it is read)."""
+    if not grouped_swiglu_bwd_supported(dy, w_down, x_up, srw, dx_up, fwd_act, dprob, dy_is_unsorted=row_sources is not None):
         raise ValueError("unsupported operands for the fused dgrad + SwiGLU backward (see grouped_swiglu_bwd_supported)")
     E, d, F = w_down.shape
-    TK = dy.shape[0]
+    TK = x_up.shape[0]
+    if row_sources is not None and not _row_sources_ok(row_sources, TK):
+        raise ValueError(f"row_sources must be a contiguous int32 CUDA tensor with {TK} elements")
     cptr, ws, nbytes = _plan_or_workspace(plan, counts, E, TK, dy.device)
     part_bytes = int(lib().fx_grouped_swiglu_bwd_ws_bytes(TK, F))
     part = torch.empty(part_bytes // 4, dtype=torch.float32, device=dy.device)
@@ -199,7 +238,7 @@ def flextrain_grouped_gemm_rows_swiglu_bwd(dy, w_down, counts, x_up, srw, dx_up,
         ptr(dy), dy.stride(0), ptr(w_down), F, w_down.stride(0), 0, ptr(x_up), x_up.stride(0), ptr(srw),
         dtype_enum(srw.dtype), ptr(dx_up), dx_up.stride(0), ptr(fwd_act), fwd_act.stride(0) if fwd_act is not None else 0,
         ptr(dprob), dtype_enum(dprob.dtype), cptr, E, TK, F, d, dtype_enum(dy.dtype), ptr(ws), nbytes, ptr(part),
-        part_bytes, stream_ptr(dy.device))
+        part_bytes, ptr(row_sources), dy.shape[0], stream_ptr(dy.device))
     check(rc, "fx_grouped_gemm_rows_swiglu_bwd")
     return dx_up, dprob, fwd_act
 

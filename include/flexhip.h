@@ -290,10 +290,16 @@ int fx_grouped_gemm_rows(const void* A, int64_t lda, const void* B, int64_t ldb,
 
 /* The per-expert weight-gradient GEMMs (flextrain/ops/full_moe.py:602-611, :617-626):
  *   G[e][M, N] = alpha * A_e[c_e, M]^T * B_e[c_e, N] + beta * G[e],  G[e] = G + e * g_expert_stride.
- * g_dt may be fp32 for bf16 inputs. */
+ * g_dt may be fp32 for bf16 inputs.
+ * a_row_map / b_row_map (optional, at most one; total_rows entries from fx_moe_row_sources): that
+ * operand is then the UNSORTED (a_rows or b_rows, M or N) activation matrix and its expert-sorted row
+ * r is row map[r] of it: the tile loads gather the rows along the contraction, and the scatter launch
+ * of flextrain/ops/moe_backend.py:440-452 with its expert-sorted copy is not needed for this product.
+ * rows * ld * 2 bytes must stay below 4 GB; map entries are clamped to the source's rows. */
 int fx_grouped_gemm_wgrad(const void* A, int64_t lda, const void* B, int64_t ldb, void* G, int64_t ldg,
                           int64_t g_expert_stride, int g_dt, const int32_t* counts, int E, int64_t total_rows,
                           int M, int N, float alpha, float beta, int dt, void* ws, size_t ws_bytes,
+                          const int32_t* a_row_map, int64_t a_rows, const int32_t* b_row_map, int64_t b_rows,
                           hipStream_t stream);
 
 /* The expert up-projection with the SwiGLU fused into its epilogue: one launch for the GEMM of
@@ -329,7 +335,9 @@ int fx_grouped_gemm_rows_glu(const void* A, int64_t lda, const void* B, int64_t 
  * K = d_model, F = expert width; trans_b as fx_grouped_gemm_rows (w_down stored (E, d, F): 0).
  * part_ws: fx_grouped_swiglu_bwd_ws_bytes(total_rows, F) bytes, 16-byte aligned.
  * Needs the 256-row tile form (fx_grouped_rows_tile_height(E, total_rows) == 256), K, F and all
- * row strides multiples of 8. */
+ * row strides multiples of 8.
+ * dy_row_map (optional): dy is then the UNSORTED (dy_rows, K) upstream gradient and expert-sorted row
+ * r is row dy_row_map[r] of it, gathered by the tile loads (as a_row_map of fx_grouped_gemm_rows_glu). */
 int fx_grouped_rows_tile_height(int E, int64_t total_rows);
 size_t fx_grouped_swiglu_bwd_ws_bytes(int64_t total_rows, int F);
 int fx_grouped_gemm_rows_swiglu_bwd(const void* dy, int64_t lddy, const void* w_down, int64_t ldb,
@@ -337,7 +345,8 @@ int fx_grouped_gemm_rows_swiglu_bwd(const void* dy, int64_t lddy, const void* w_
                                     const void* srw, int srw_dt, void* dx_up, int64_t lddx, void* fwd_act,
                                     int64_t ldact, void* dprob, int dprob_dt, const int32_t* counts, int E,
                                     int64_t total_rows, int F, int K, int dt, void* ws, size_t ws_bytes, void* part_ws,
-                                    size_t part_ws_bytes, hipStream_t stream);
+                                    size_t part_ws_bytes, const int32_t* dy_row_map, int64_t dy_rows,
+                                    hipStream_t stream);
 
 /* Gate and up projections of the dense gated FFN with the activation in the epilogue: replaces the
  * two matmuls and the gated-activation launch of flextrain/nn/blocks/ffn_dense.py:130-146.

@@ -422,3 +422,60 @@ def test_fused_dgrad_swiglu_bwd_equals_the_two_launches(dev, E, TK, d, F, dprob_
         _close_scaled(dx[a:b], want_dx, f"dx_up of expert {e}")
         _close_scaled(act[a:b], want_act, f"saved activation of expert {e}")
         _close_scaled(dw[a:b].reshape(-1), want_dw.reshape(-1), f"router-weight gradient of expert {e}")
+
+
+@pytest.mark.parametrize("T,E,K,d,F", [(1200, 4, 2, 192, 136), (8192, 128, 8, 2048, 768)])
+def test_backward_launches_gather_unsorted_rows_bit_for_bit(dev, T, E, K, d, F):
+    """The expert backward without expert-sorted copies of dy and x: the fused dgrad launch (rows of
+    the unsorted upstream gradient through the row map) and both weight-gradient launches (unsorted
+    operand gathered along the contraction, as A and as B) against the same launches on the scattered
+    copies.  Same values reach the same MFMAs in the same order: every output must match bit for bit."""
+    from flextrain_amd.ops import moe as moe_ops
+    from flextrain_amd.ops.grouped import flextrain_grouped_gemm_rows_swiglu_bwd
+
+    g = gen(T + E)
+    TK = T * K
+    logits = torch.randn(T, E, generator=g)
+    ids = logits.topk(K, dim=1).indices.to(torch.int32).to(dev)
+    mapping, counts = moe_ops.flextrain_moe_sort(ids, num_experts=E)
+    src = moe_ops.flextrain_moe_row_sources(mapping)
+    dy, x = randn(g, T, d, std=0.5).to(dev), randn(g, T, d, std=0.5).to(dev)
+    sdy, sx = torch.empty(TK, d, dtype=torch.bfloat16, device=dev), torch.empty(TK, d, dtype=torch.bfloat16, device=dev)
+    moe_ops.flextrain_moe_scatter(dy, mapping, out=sdy)
+    moe_ops.flextrain_moe_scatter(x, mapping, out=sx)
+    w_down = randn(g, E, d, F, std=0.1).to(dev)
+    x_up = randn(g, TK, 2 * F).to(dev)
+    srw = torch.rand(TK, 1, generator=g).to(torch.bfloat16).to(dev)
+
+    def fused(dy_arg, rows):
+        dx = torch.full((TK, 2 * F), 7.0, dtype=torch.bfloat16, device=dev)
+        act = torch.full((TK, F), 7.0, dtype=torch.bfloat16, device=dev)
+        dw = torch.full((TK, 1), 7.0, dtype=torch.bfloat16, device=dev)
+        flextrain_grouped_gemm_rows_swiglu_bwd(dy_arg, w_down, counts, x_up, srw, dx, dw, fwd_act=act, row_sources=rows)
+        return dx, act, dw
+
+    for got, want, what in zip(fused(dy, src), fused(sdy, None), ("dx_up", "saved activation", "router-weight gradient")):
+        assert torch.equal(got, want), f"{what}: {int((got != want).sum())} of {got.numel()} elements differ"
+    dx_up = fused(sdy, None)[0]
+    act = fused(sdy, None)[1]
+    for gdt in (torch.bfloat16, torch.float32):
+        g0 = randn(g, E, d, F, dtype=gdt).to(dev)
+        ga, gb = g0.clone(), g0.clone()
+        flextrain_grouped_gemm_wgrad(sdy, act, ga, counts)                              # g_down, sorted A
+        flextrain_grouped_gemm_wgrad(dy, act, gb, counts, a_row_sources=src)            # g_down, gathered A
+        assert torch.equal(ga, gb), f"g_down ({gdt}): {int((ga != gb).sum())} elements differ"
+        g1 = randn(g, E, 2 * F, d, dtype=gdt).to(dev)
+        ga, gb = g1.clone(), g1.clone()
+        flextrain_grouped_gemm_wgrad(dx_up, sx, ga, counts)                             # g_up, sorted B
+        flextrain_grouped_gemm_wgrad(dx_up, x, gb, counts, b_row_sources=src)           # g_up, gathered B
+        assert torch.equal(ga, gb), f"g_up ({gdt}): {int((ga != gb).sum())} elements differ"
+    # a map with entries outside the source is clamped, never followed out of bounds
+    bad = src.clone()
+    bad[::5] = 1 << 30
+    bad[1::7] = -3
+    gc, gd = g1.clone(), g1.clone()
+    flextrain_grouped_gemm_wgrad(dx_up, x, gc, counts, b_row_sources=bad)
+    flextrain_grouped_gemm_wgrad(dx_up, x, gd, counts, b_row_sources=bad.clamp(0, T - 1))
+    assert torch.equal(gc, gd) and bool(torch.isfinite(gc.float()).all())
+    with pytest.raises(ValueError):
+        flextrain_grouped_gemm_wgrad(dy, x, g1, counts, a_row_sources=src, b_row_sources=src)
