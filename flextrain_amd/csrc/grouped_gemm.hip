@@ -422,8 +422,14 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void grouped_wgrad_walk_ker
         Tile t;
         t.e = p / tiles_per_expert;
         const int q = p % tiles_per_expert;
-        t.tm = q / tiles_n;
-        t.tn = q % tiles_n;
+        if (KG == 2) {          // consecutive tiles share the gathered operand's tile (20 us of 680 at 128 experts x 512 rows)
+            const int tiles_m = tiles_per_expert / tiles_n;
+            t.tn = q / tiles_m;
+            t.tm = q % tiles_m;
+        } else {
+            t.tm = q / tiles_n;
+            t.tn = q % tiles_n;
+        }
         t.row0 = OFFSETS[t.e];
         t.rows = OFFSETS[t.e + 1] - OFFSETS[t.e];
         return t;
