@@ -73,7 +73,7 @@ def _parse():
     ap.add_argument("--no-extra", action="store_true", help="skip the non-headline configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--only", default="", help="comma-separated subset of the non-headline configurations "
-                                               "(c1, c3, c4, c5, ffn, attn, act, disp, probe) to run, e.g. for a profiler pass")
+                                               "(c1, c3, c4, c5, moe_ref, ffn, attn, act, disp, probe) to run, e.g. for a profiler pass")
     return ap.parse_args()
 
 
@@ -156,6 +156,8 @@ def run_extra(torch, ops, dev, stream, rn, only):
         rows += run_lm_head(torch, dev, stream, rn)
     if want("c5"):
         rows += run_moe(torch, dev, stream, rn)
+    if want("moe_ref"):
+        rows += _moe_reference_microbench(torch, dev, stream, rn)
     if want("ffn"):
         rows += run_ffn_dense(torch, dev, stream, rn)
     if want("attn"):
@@ -766,7 +768,6 @@ def run_moe(torch, dev, stream, rn):
     del sx, act, x, dy, out, weights, grads, slot
     pool.clear()
     torch.cuda.empty_cache()
-    rows += _moe_reference_microbench(torch, dev, stream, rn)
     return rows
 
 
