@@ -994,14 +994,20 @@ def main():
         rec("swiglu_bwd", lambda: ops.flextrain_swiglu_bwd(gate, up, dout, dx1=dgate, dx3=dup))
         ops.flextrain_rope_bwd([qs[j], ks[j]], pos, inv_freq)
 
-    # one plain copy of known size (reads and writes 234,881,024 bytes each): the yardstick that hardware
-    # counter runs of this script scale FETCH_SIZE / WRITE_SIZE by
-    out.copy_(gate)
+    # One plain pass of known size (reads and writes 536,870,912 bytes each, as an elementwise NOT so that
+    # the launch has a kernel name of its own in a trace): the yardstick that hardware counter runs of
+    # this script scale FETCH_SIZE / WRITE_SIZE by.  Larger than the 256 MB last-level cache and issued
+    # after the warm-up steps have streamed gigabytes through it, so that its source is read from HBM
+    # (a copy of a buffer that was just written is served from that cache and reads ~0).
+    calib_src = torch.zeros(512 << 20, dtype=torch.uint8, device=dev)
+    calib_dst = torch.empty_like(calib_src)
     untimed = lambda name, fn: fn()
     with torch.cuda.stream(stream):
         for _ in range(args.warmup):
             step(untimed)
+        torch.bitwise_not(calib_src, out=calib_dst)
         torch.cuda.synchronize()
+        del calib_src, calib_dst
         t0 = time.perf_counter()
         for _ in range(args.steps):
             step(timed)
