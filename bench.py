@@ -144,30 +144,38 @@ def _time_launches(torch, stream, fns, warmup=5, reps=20, settle_ms=40.0, window
     return a.elapsed_time(b) / reps
 
 
+def _progress(text):
+    """One line on stderr per leg, flushed before the leg touches the GPU: what a run that dies leaves behind."""
+    print(f"[bench {time.strftime('%H:%M:%S')}] {text}", file=sys.stderr, flush=True)
+
+
 def run_extra(torch, ops, dev, stream, rn, only):
+    """The legs beside the headline workload.  A leg that raises is recorded as a row with its error
+    and ends the GPU legs (a failed launch leaves the context unusable); the rows measured so far and
+    the headline figure are still reported."""
     want = lambda tag: not only or tag in only
+    legs = (("c1", lambda: run_rmsnorm(torch, ops, dev, stream, rn)),
+            ("c4", lambda: run_adamw(torch, ops, dev, stream) + run_streamed_adamw(torch, dev)),
+            ("c3", lambda: run_lm_head(torch, dev, stream, rn)),
+            ("c5", lambda: run_moe(torch, dev, stream, rn)),
+            ("moe_ref", lambda: _moe_reference_microbench(torch, dev, stream, rn)),
+            ("ffn", lambda: run_ffn_dense(torch, dev, stream, rn)),
+            ("attn", lambda: run_attention_proj(torch, dev, stream, rn)),
+            ("act", lambda: run_activation_slots(torch, dev)),
+            ("disp", lambda: run_dispatch_overhead(torch, dev, stream)),
+            ("probe", lambda: run_hw_probe(torch, dev)))
     rows = []
-    if want("c1"):
-        rows += run_rmsnorm(torch, ops, dev, stream, rn)
-    if want("c4"):
-        rows += run_adamw(torch, ops, dev, stream)
-        rows += run_streamed_adamw(torch, dev)
-    if want("c3"):
-        rows += run_lm_head(torch, dev, stream, rn)
-    if want("c5"):
-        rows += run_moe(torch, dev, stream, rn)
-    if want("moe_ref"):
-        rows += _moe_reference_microbench(torch, dev, stream, rn)
-    if want("ffn"):
-        rows += run_ffn_dense(torch, dev, stream, rn)
-    if want("attn"):
-        rows += run_attention_proj(torch, dev, stream, rn)
-    if want("act"):
-        rows += run_activation_slots(torch, dev)
-    if want("disp"):
-        rows += run_dispatch_overhead(torch, dev, stream)
-    if want("probe"):
-        rows += run_hw_probe(torch, dev)
+    for tag, leg in legs:
+        if not want(tag):
+            continue
+        _progress(f"leg {tag}")
+        try:
+            rows += leg()
+            torch.cuda.synchronize()
+        except Exception as exc:  # noqa: BLE001 - reported in the output line, not swallowed
+            _progress(f"leg {tag} FAILED: {type(exc).__name__}: {exc}")
+            rows.append({"op": f"{tag}.FAILED", "unit": "", "error": f"{type(exc).__name__}: {exc}"[:400]})
+            break
     return rows
 
 
@@ -954,8 +962,13 @@ def main():
     lib()  # fail loudly before any timing if the native library is missing
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    # Every launch of this script, torch's and the library's, goes to ONE stream, made current here for
+    # the whole run: inputs are produced on the stream that the timed launches consume them on, so no
+    # launch can overtake the kernel that writes its operands (routing tables, labels, weights).
     stream = torch.cuda.Stream(device=dev)
+    torch.cuda.set_stream(stream)
     timed = Timed(torch, stream)
+    _progress("headline workload: inputs")
 
     # ------------------------------------------------------------------ inputs
     T, HQ, HK, HD, F = 8192, 32, 8, 128, 14336
@@ -1002,6 +1015,7 @@ def main():
     calib_src = torch.zeros(512 << 20, dtype=torch.uint8, device=dev)
     calib_dst = torch.empty_like(calib_src)
     untimed = lambda name, fn: fn()
+    _progress("headline workload: warm-up, calibration pass, timed steps")
     with torch.cuda.stream(stream):
         for _ in range(args.warmup):
             step(untimed)
@@ -1051,11 +1065,14 @@ def main():
     mfma_probe = None
     if not args.no_extra:
         op_rows += run_extra(torch, ops, dev, stream, rn, [t.strip() for t in args.only.split(",") if t.strip()])
-        mfma_probe = run_mfma_probe(torch, dev, stream)
-        for row in op_rows:
-            if row["unit"] == "TFLOP/s":
-                row["frac_of_sustained_mfma_random_operands"] = round(
-                    row["achieved"] / mfma_probe["random_operands"]["tflops"], 4)
+        if not any("error" in r for r in op_rows):
+            _progress("mfma probe")
+            mfma_probe = run_mfma_probe(torch, dev, stream)
+            for row in op_rows:
+                if row["unit"] == "TFLOP/s":
+                    row["frac_of_sustained_mfma_random_operands"] = round(
+                        row["achieved"] / mfma_probe["random_operands"]["tflops"], 4)
+    _progress("cpu baselines")
 
     # -------------------------------------------------------- CPU baseline
     cpu = None
@@ -1137,6 +1154,7 @@ def main():
         brief("ffn.down gemm [", "ffn.down"), brief("ffn.down gemm, vendor", "ffn.down vendor"),
         brief("ffn.dense block fwd+bwd", "ffn.block"), brief("attn.projections fwd+bwd", "attn.proj"),
         brief("probe.save-level", "gemm8192^3")) if t is not None]
+    summary += [f"{r['op']}: {r['error']}" for r in op_rows if "error" in r]
 
     result = {
         "metric": METRIC,

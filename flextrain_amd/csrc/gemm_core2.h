@@ -410,7 +410,7 @@ struct TileLoaderKG {
 #pragma unroll
         for (int j = 0; j < NI; ++j) {
             const int kk = min(kpos + j * NW * KPI, kext - 1);
-            nidx[j] = kmap[kk < 0 ? 0 : kk];
+            nidx[j] = kk >= 0 ? kmap[kk] : 0;       // an empty group has no map entry to read (its map may end the buffer)
         }
         kpos += GEMM_BK;
     }
