@@ -322,7 +322,7 @@ extern "C" int fx_softmax_ce(const void* logits, void* dz_out, const void* label
     if (!(softcap >= 0.f)) FX_FAIL("fx_softmax_ce: softcap must be 0 (off) or positive");
     if (rows == 0) return 0;
     if (!logits || !dz_out || !labels || !loss_out) FX_FAIL("fx_softmax_ce: null pointer");
-    if (in_row_stride < V || out_row_stride < V) FX_FAIL("fx_softmax_ce: a row stride is smaller than the row");
+    if (rows > 1 && (in_row_stride < V || out_row_stride < V)) FX_FAIL("fx_softmax_ce: a row stride is smaller than the row");
     const bool vec = (V % 8 == 0) && (in_row_stride % 8 == 0) && (out_row_stride % 8 == 0) && aligned16(logits) && aligned16(dz_out);
 #define FX_SMCE(TT, TL, CAP_)                                                                                         \
     softmax_ce_kernel<TT, TL, CAP_><<<(unsigned)rows, SM_THREADS, 0, stream>>>(                                        \
@@ -348,7 +348,7 @@ extern "C" int fx_softcap_fwd(void* logits, void* gate_out, int64_t rows, int V,
     if (!(softcap > 0.f)) FX_FAIL("fx_softcap_fwd: softcap must be positive");
     if (rows == 0) return 0;
     if (!logits || !gate_out) FX_FAIL("fx_softcap_fwd: null pointer");
-    if (row_stride < V || gate_row_stride < V) FX_FAIL("fx_softcap_fwd: a row stride is smaller than the row");
+    if (rows > 1 && (row_stride < V || gate_row_stride < V)) FX_FAIL("fx_softcap_fwd: a row stride is smaller than the row");
     const bool vec = (V % 8 == 0) && (row_stride % 8 == 0) && (gate_row_stride % 8 == 0) && aligned16(logits) && aligned16(gate_out);
     FX_DISPATCH_DTYPE(dt, TT,
         softcap_fwd_kernel<TT><<<flat_grid(rows * (vec ? V / 8 : V)), 256, 0, stream>>>(
@@ -362,7 +362,7 @@ extern "C" int fx_softcap_bwd(void* dz, const void* gate, int64_t rows, int V, i
     if (rows < 0 || V <= 0) FX_FAIL("fx_softcap_bwd: bad shape");
     if (rows == 0) return 0;
     if (!dz || !gate) FX_FAIL("fx_softcap_bwd: null pointer");
-    if (row_stride < V || gate_row_stride < V) FX_FAIL("fx_softcap_bwd: a row stride is smaller than the row");
+    if (rows > 1 && (row_stride < V || gate_row_stride < V)) FX_FAIL("fx_softcap_bwd: a row stride is smaller than the row");
     const bool vec = (V % 8 == 0) && (row_stride % 8 == 0) && (gate_row_stride % 8 == 0) && aligned16(dz) && aligned16(gate);
     FX_DISPATCH_DTYPE(dt, TT,
         softcap_bwd_kernel<TT><<<flat_grid(rows * (vec ? V / 8 : V)), 256, 0, stream>>>(
