@@ -37,7 +37,8 @@ typedef struct ihipStream_t* hipStream_t;
 #define FX_ACT_SILU 0
 #define FX_ACT_GELU_TANH 1
 
-/* Library identification: returns a static string "flexhip <version> gfx950". */
+/* Library identification: returns a static string "flexhip <version> gfx950".  No counterpart in the
+ * reference (its kernels are Python functions); lets a binding check what it loaded. */
 const char* fx_version(void);
 
 /* ---- RMSNorm ----------------------------------------------------------- */
@@ -261,7 +262,9 @@ int fx_softcap_bwd(void* dz, const void* gate, int64_t rows, int V, int64_t row_
 
 /* ---- Expert-grouped GEMMs -------------------------------------------------- */
 
-/* Scratch bytes for the grouped GEMM entry points (row offsets + tile list). */
+/* Scratch bytes for the grouped GEMM entry points (plan header, row offsets, tile list).  No counterpart
+ * in the reference, whose per-expert loop (flextrain/ops/full_moe.py:428-626) slices on the host: here the
+ * offsets and tiles are built on the device from the counts, and the caller lends the memory. */
 size_t fx_grouped_ws_bytes(int E, int64_t total_rows);
 
 /* Row offsets and tile list of one routing, made once and shared by several grouped launches: a
@@ -427,7 +430,8 @@ int fx_copy_fields(int n, void* const* dst, const void* const* src, const int64_
                    int direction, hipStream_t stream);
 
 /* Device staging bytes fx_adamw_stream_chunk needs for n_slots slots of sub_elems
- * elements (p, g, m, v and, when stage_bf16_copy, the bf16 copy of p). */
+ * elements (p, g, m, v and, when stage_bf16_copy, the bf16 copy of p): the role of the reference's
+ * optimizer ring slots (flextrain/engine/buffers.py:1088-1291), sized by the caller there. */
 size_t fx_adamw_stream_ws_bytes(int64_t sub_elems, int n_slots, int p_dt, int g_dt, int state_dt,
                                 int stage_bf16_copy);
 
