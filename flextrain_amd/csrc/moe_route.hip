@@ -225,7 +225,11 @@ __global__ __launch_bounds__(SORT_CHUNK) void sort_map_kernel(const TI* __restri
     const int e = i < n ? (int)IDS[i] : -1;
     ids[threadIdx.x] = e;
     __syncthreads();
-    if (i >= n || e < 0 || e >= E) return;
+    if (i >= n) return;
+    if (e < 0 || e >= E) {     // not counted by the histogram: give the pair a row inside the buffers, so that
+        MAP[i] = (TO)0;        // a scatter or gather through this map cannot leave them
+        return;
+    }
     int rank = 0;
     const int4* v = reinterpret_cast<const int4*>(ids);
     const int me = threadIdx.x;

@@ -144,7 +144,9 @@ size_t fx_moe_sort_ws_bytes(int64_t n_pairs, int E);
  * flextrain_copy_expert_counts (:787-834).  ids: n_pairs = T*K flat expert ids
  * (int32, or int64 when ids_are_int64).  index_out[i] = row of pair i in the
  * expert-grouped order (stable).  counts_out (device, E int32) and counts_host
- * (pinned host memory mapped into the device, E int32) are optional. */
+ * (pinned host memory mapped into the device, E int32) are optional.  An id outside [0, E) is a
+ * caller error the reference does not define: here it is not counted and its pair is mapped to
+ * row 0, so that scatters and gathers through the map stay inside their buffers. */
 int fx_moe_sort(const void* ids, int ids_are_int64, int64_t n_pairs, int E, void* index_out,
                 int index_is_int64, int32_t* counts_out, int32_t* counts_host, void* ws, size_t ws_bytes,
                 hipStream_t stream);

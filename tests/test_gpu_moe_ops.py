@@ -95,6 +95,27 @@ def test_sort_bit_exact(dev, T, K, E, idt):
     assert torch.equal(torch.sort(mapping.reshape(-1).cpu().long()).values, torch.arange(T * K))
 
 
+def test_sort_maps_ids_outside_the_expert_range_to_row_zero(dev):
+    """A caller error the reference leaves undefined: such a pair is not counted, and its map entry is 0 (inside
+    every buffer) instead of whatever the output held; the valid pairs keep the stable order among themselves."""
+    g = gen(1011)
+    T, K, E = 512, 4, 16
+    ids = torch.randint(0, E, (T, K), generator=g, dtype=torch.int32)
+    bad = torch.rand(T, K, generator=g) < 0.05
+    ids[bad] = torch.where(torch.rand(int(bad.sum()), generator=g) < 0.5, -3, E + 5).to(torch.int32)
+    out = torch.full((T, K), 1 << 30, dtype=torch.int32, device=dev)
+    mapping, counts = ops.flextrain_moe_sort(ids.to(dev), E, indices=out)
+    flat, ok = ids.reshape(-1), ~bad.reshape(-1)
+    cnt_ref = torch.bincount(flat[ok].long(), minlength=E).to(torch.int32)
+    assert torch.equal(counts.cpu(), cnt_ref)
+    m = mapping.reshape(-1).cpu().long()
+    assert bool((m[~ok] == 0).all())
+    order = torch.argsort(flat[ok].long(), stable=True)          # valid pairs, grouped by expert, first come first
+    want = torch.empty_like(order)
+    want[order] = torch.arange(order.numel())
+    assert torch.equal(m[ok], want)
+
+
 def test_sort_slot_buffers_and_copy_counts(dev):
     g = gen(6)
     ids = torch.randint(0, 16, (100, 4), generator=g, dtype=torch.int32)
