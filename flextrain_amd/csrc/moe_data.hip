@@ -13,8 +13,12 @@
 
 namespace fx {
 
-FX_DEV int64_t load_index(const void* idx, int is64, int64_t i) {
-    return is64 ? reinterpret_cast<const int64_t*>(idx)[i] : (int64_t)reinterpret_cast<const int32_t*>(idx)[i];
+// Entry i of an index mapping, clamped to [0, rows): a mapping that is no permutation of the routed
+// rows (a caller's own, or one made from expert ids outside the range) moves the wrong rows, never
+// an address outside the buffers.
+FX_DEV int64_t load_index(const void* idx, int is64, int64_t i, int64_t rows) {
+    const int64_t r = is64 ? reinterpret_cast<const int64_t*>(idx)[i] : (int64_t)reinterpret_cast<const int32_t*>(idx)[i];
+    return r < 0 ? 0 : (r < rows ? r : rows - 1);
 }
 
 // ------------------------------------------------------------------ scatter
@@ -32,7 +36,7 @@ __global__ __launch_bounds__(256) void moe_scatter_kernel(
             float v[8];
             load_f32<T, 8>(X + t * D + c, v);
             for (int k = 0; k < K; ++k) {
-                const int64_t row = load_index(IDX, idx64, t * K + k);
+                const int64_t row = load_index(IDX, idx64, t * K + k, Tn * K);
                 if (HAS_SCALE) {
                     const float s = (float)SCALE[t * K + k];
                     float o[8];
@@ -48,7 +52,7 @@ __global__ __launch_bounds__(256) void moe_scatter_kernel(
         for (int c = lane; c < D; c += tpt) {
             const float v = (float)X[t * D + c];
             for (int k = 0; k < K; ++k) {
-                const int64_t row = load_index(IDX, idx64, t * K + k);
+                const int64_t row = load_index(IDX, idx64, t * K + k, Tn * K);
                 OUT[row * out_stride + c] = HAS_SCALE ? (T)(v * (float)SCALE[t * K + k]) : X[t * D + c];
             }
         }
@@ -60,7 +64,7 @@ __global__ __launch_bounds__(256) void moe_scatter_weights_kernel(const T* __res
                                                                   const void* __restrict__ IDX, int idx64,
                                                                   T* __restrict__ OUT, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i < n) OUT[load_index(IDX, idx64, i)] = W[i];
+    if (i < n) OUT[load_index(IDX, idx64, i, n)] = W[i];
 }
 
 // ------------------------------------------------------------------- gather
@@ -89,7 +93,7 @@ __global__ __launch_bounds__(256) void moe_gather_kernel(
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     if (k0 + u < K) {
-                        const int64_t row = load_index(IDX, idx64, t * K + k0 + u);
+                        const int64_t row = load_index(IDX, idx64, t * K + k0 + u, Tn * K);
                         load_f32<T, 8>(Y + row * D + c, v[u]);
                         w[u] = W != nullptr ? (float)W[t * K + k0 + u] : 1.f;
                     }
@@ -113,7 +117,7 @@ __global__ __launch_bounds__(256) void moe_gather_kernel(
         for (int c = lane; c < D; c += tpt) {
             float acc = RES != nullptr ? (float)RES[t * D + c] : 0.f;
             for (int k = 0; k < K; ++k) {
-                const int64_t row = load_index(IDX, idx64, t * K + k);
+                const int64_t row = load_index(IDX, idx64, t * K + k, Tn * K);
                 const float v = (float)Y[row * D + c];
                 acc += W != nullptr ? v * (float)W[t * K + k] : v;
             }

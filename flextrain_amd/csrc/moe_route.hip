@@ -251,6 +251,13 @@ __global__ __launch_bounds__(256) void copy_i32_kernel(const int32_t* __restrict
 // ---------------------------------------------------------------------------
 // Router backward (one wave per token).
 // ---------------------------------------------------------------------------
+// Row of pair i in the expert-sorted buffers, clamped to them (see load_index in moe_data.hip).
+template <typename TI>
+FX_DEV int64_t pair_row(const TI* __restrict__ indices, int64_t i, int64_t rows) {
+    const int64_t r = (int64_t)indices[i];
+    return r < 0 ? 0 : (r < rows ? r : rows - 1);
+}
+
 template <typename T, typename TDP, typename TI, int MODE>
 __global__ __launch_bounds__(256) void router_gate_bwd_kernel(
     T* __restrict__ DLOGITS, const TDP* __restrict__ DPROBS, const T* __restrict__ PROBS,
@@ -263,11 +270,11 @@ __global__ __launch_bounds__(256) void router_gate_bwd_kernel(
         // dz_k = p_k (dp_k - sum_j p_j dp_j), added into dlogits[t, expert_k]
         float dot = 0.f;
         for (int k = lane; k < K; k += 64)
-            dot += (float)DPROBS[(int64_t)INDICES[t * K + k]] * (float)PROBS[t * K + k];
+            dot += (float)DPROBS[pair_row(INDICES, t * K + k, Tn * K)] * (float)PROBS[t * K + k];
         dot = group_sum<64>(dot);
         for (int k = lane; k < K; k += 64) {
             const float p = (float)PROBS[t * K + k];
-            const float dp = (float)DPROBS[(int64_t)INDICES[t * K + k]];
+            const float dp = (float)DPROBS[pair_row(INDICES, t * K + k, Tn * K)];
             const int e = EXPERTS[t * K + k];
             if (e >= 0 && e < E) {
                 T* o = DLOGITS + t * E + e;
@@ -286,14 +293,14 @@ __global__ __launch_bounds__(256) void router_gate_bwd_kernel(
         for (int k = lane; k < K; k += 64) {
             const int e = EXPERTS[t * K + k];
             if (e >= 0 && e < E)
-                row_dot += (float)DPROBS[(int64_t)INDICES[t * K + k]] * (expf((float)LOGITS[t * E + e] - mx) / sum);
+                row_dot += (float)DPROBS[pair_row(INDICES, t * K + k, Tn * K)] * (expf((float)LOGITS[t * E + e] - mx) / sum);
         }
         row_dot = group_sum<64>(row_dot);
         for (int e = lane; e < E; e += 64) {
             const float p = expf((float)LOGITS[t * E + e] - mx) / sum;
             float dz = -p * row_dot;
             for (int k = 0; k < K; ++k)
-                if (EXPERTS[t * K + k] == e) dz += (float)DPROBS[(int64_t)INDICES[t * K + k]] * p;
+                if (EXPERTS[t * K + k] == e) dz += (float)DPROBS[pair_row(INDICES, t * K + k, Tn * K)] * p;
             T* o = DLOGITS + t * E + e;
             *o = (T)((float)*o + round_to<T>(dz));
         }

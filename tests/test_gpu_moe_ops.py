@@ -116,6 +116,19 @@ def test_sort_maps_ids_outside_the_expert_range_to_row_zero(dev):
     assert torch.equal(m[ok], want)
 
 
+def test_gather_clamps_a_mapping_that_leaves_the_buffer(dev):
+    """A caller's own mapping with entries outside the routed rows reads the clamped rows, never past the buffer."""
+    g = gen(1012)
+    T, K, D = 64, 2, 64
+    y = randn(g, T * K, D).to(dev)
+    mapping = torch.randperm(T * K, generator=g).view(T, K).to(torch.int32)
+    bad = mapping.clone()
+    bad[3, 1], bad[10, 0], bad[63, 1] = 1 << 28, -7, T * K
+    clamped = bad.clamp(0, T * K - 1)
+    assert torch.equal(ops.flextrain_moe_gather(y, bad.to(dev)), ops.flextrain_moe_gather(y, clamped.to(dev)))
+    assert torch.equal(ops.flextrain_moe_gather(y, bad.long().to(dev)), ops.flextrain_moe_gather(y, clamped.to(dev)))
+
+
 def test_sort_slot_buffers_and_copy_counts(dev):
     g = gen(6)
     ids = torch.randint(0, 16, (100, 4), generator=g, dtype=torch.int32)
