@@ -23,6 +23,14 @@ def pytest_sessionstart(session):
         __graft_entry__.build()
 
 
+def pytest_runtest_setup(item):
+    """Name every GPU test on the real stderr, flushed, before it touches the card: a run that ends with
+    the machine (a fault takes the box and its files along) still shows which test it was in."""
+    if item.get_closest_marker("gpu") is not None:
+        sys.__stderr__.write(f"[gpu test] {item.nodeid}\n")
+        sys.__stderr__.flush()
+
+
 @pytest.fixture(scope="session")
 def dev():
     if not torch.cuda.is_available():
