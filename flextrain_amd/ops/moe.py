@@ -19,6 +19,29 @@ def _routing_mode_id(mode: str) -> int:
     raise ValueError(f"unknown routing mode: {mode!r}")
 
 
+def _on_gpu(**tensors) -> None:
+    """ValueError for a given tensor that is not on the GPU (None entries are optional arguments not given)."""
+    for name, t in tensors.items():
+        if t is not None and not t.is_cuda:
+            raise ValueError(f"{name} must be a CUDA tensor")
+
+
+def _dense(**tensors) -> None:
+    for name, t in tensors.items():
+        if t is not None and not t.is_contiguous():
+            raise ValueError(f"{name} must be contiguous")
+
+
+def _shaped(t, name, *shape) -> None:
+    if tuple(t.shape) != shape:
+        raise ValueError(f"{name} is {tuple(t.shape)}, expected {shape}")
+
+
+def _counted(t, name, n, what="") -> None:
+    if t.numel() != n:
+        raise ValueError(f"{name} holds {t.numel()} elements, expected {n}{what}")
+
+
 def _is64(t: torch.Tensor) -> int:
     if t.dtype == torch.int64:
         return 1
@@ -31,33 +54,27 @@ def flextrain_fused_topk_softmax(gate_logits, top_k, topk_ids_out=None, topk_wei
                                  mode="topk_then_softmax"):
     """-> ``(topk_weights [T,K], topk_ids [T,K] int32)``;
     flextrain/ops/_kernels/moe.py:848-943."""
-    if not gate_logits.is_cuda:
-        raise ValueError("gate_logits must be a CUDA tensor")
-    if not gate_logits.is_contiguous():
-        raise ValueError("gate_logits must be contiguous")
+    _on_gpu(gate_logits=gate_logits)
+    _dense(gate_logits=gate_logits)
     if gate_logits.dim() != 2:
-        raise ValueError(f"gate_logits must be 2D, got {gate_logits.dim()}D")
+        raise ValueError(f"gate_logits must be (tokens, experts), got {gate_logits.dim()} dimensions")
     T, E = gate_logits.shape
     K = top_k
     if K > E:
-        raise ValueError(f"top_k ({K}) cannot exceed num_experts ({E})")
+        raise ValueError(f"top_k = {K} with only {E} experts")
     mode_id = _routing_mode_id(mode)
     if topk_ids_out is None:
         topk_ids_out = torch.empty((T, K), dtype=torch.int32, device=gate_logits.device)
     else:
-        if tuple(topk_ids_out.shape) != (T, K):
-            raise ValueError(f"topk_ids_out shape {tuple(topk_ids_out.shape)} must be [{T}, {K}]")
-        if not topk_ids_out.is_contiguous():
-            raise ValueError("topk_ids_out must be contiguous")
+        _shaped(topk_ids_out, "topk_ids_out", T, K)
+        _dense(topk_ids_out=topk_ids_out)
         if topk_ids_out.dtype != torch.int32:
             raise TypeError("topk_ids_out must be int32")
     if topk_weights_out is None:
         topk_weights_out = torch.empty((T, K), dtype=gate_logits.dtype, device=gate_logits.device)
     else:
-        if tuple(topk_weights_out.shape) != (T, K):
-            raise ValueError(f"topk_weights_out shape {tuple(topk_weights_out.shape)} must be [{T}, {K}]")
-        if not topk_weights_out.is_contiguous():
-            raise ValueError("topk_weights_out must be contiguous")
+        _shaped(topk_weights_out, "topk_weights_out", T, K)
+        _dense(topk_weights_out=topk_weights_out)
     rc = lib().fx_topk_softmax(ptr(gate_logits), ptr(topk_ids_out), ptr(topk_weights_out), T, E, K,
                                dtype_enum(gate_logits.dtype), dtype_enum(topk_weights_out.dtype), mode_id,
                                stream_ptr(gate_logits.device))
@@ -72,8 +89,7 @@ def flextrain_moe_sort(topk_ids, num_experts, indices=None, expert_counts_gpu=No
     signature compatibility and ignored.  ``expert_counts_pinned`` (extension):
     a pinned int32 host tensor that the sort fills directly, which saves the
     separate :func:`flextrain_copy_expert_counts` launch."""
-    if not topk_ids.is_cuda:
-        raise ValueError("topk_ids must be a CUDA tensor")
+    _on_gpu(topk_ids=topk_ids)
     flat_ids = topk_ids.flatten()
     if not flat_ids.is_contiguous():
         flat_ids = flat_ids.contiguous()
@@ -83,12 +99,9 @@ def flextrain_moe_sort(topk_ids, num_experts, indices=None, expert_counts_gpu=No
         indices_flat = torch.empty_like(flat_ids)
         result = indices_flat.view(topk_ids.shape)
     else:
-        if indices.shape != topk_ids.shape:
-            raise ValueError(f"indices shape {indices.shape} must match topk_ids shape {topk_ids.shape}")
-        if not indices.is_cuda:
-            raise ValueError("indices must be a CUDA tensor")
-        if not indices.is_contiguous():
-            raise ValueError("indices must be contiguous")
+        _shaped(indices, "indices", *topk_ids.shape)
+        _on_gpu(indices=indices)
+        _dense(indices=indices)
         indices_flat = indices
         result = indices
     total_counts = torch.empty(num_experts, dtype=torch.int32, device=dev)
@@ -112,12 +125,10 @@ def flextrain_moe_sort(topk_ids, num_experts, indices=None, expert_counts_gpu=No
 def flextrain_copy_expert_counts(gpu_counts, cpu_buffer) -> None:
     """Kernel-side store of the counts into pinned host memory; the caller
     synchronises before reading.  flextrain/ops/_kernels/moe.py:787-834."""
-    if not gpu_counts.is_cuda:
-        raise ValueError("gpu_counts must be a CUDA tensor")
+    _on_gpu(gpu_counts=gpu_counts)
     if not cpu_buffer.is_pinned():
-        raise ValueError("cpu_buffer must be pinned memory (use pin_memory=True)")
-    if gpu_counts.shape != cpu_buffer.shape:
-        raise ValueError(f"Shape mismatch: gpu_counts {gpu_counts.shape} vs cpu_buffer {cpu_buffer.shape}")
+        raise ValueError("cpu_buffer must be pinned host memory: the kernel stores into it directly")
+    _shaped(cpu_buffer, "cpu_buffer", *gpu_counts.shape)
     if gpu_counts.dtype != torch.int32 or cpu_buffer.dtype != torch.int32:
         raise TypeError("expert counts must be int32")
     rc = lib().fx_copy_i32(ptr(gpu_counts), cpu_buffer.data_ptr(), gpu_counts.numel(),
@@ -127,32 +138,18 @@ def flextrain_copy_expert_counts(gpu_counts, cpu_buffer) -> None:
 
 def flextrain_moe_scatter(x, indices, scales=None, out=None):
     """``out[indices[t,k]] = x[t] (* scales[t,k])``; flextrain/ops/_kernels/moe.py:946-1050."""
-    if not x.is_cuda:
-        raise ValueError("x must be a CUDA tensor")
-    if not indices.is_cuda:
-        raise ValueError("indices must be a CUDA tensor")
-    if not x.is_contiguous():
-        raise ValueError("x must be contiguous")
-    if not indices.is_contiguous():
-        raise ValueError("indices must be contiguous")
+    _on_gpu(x=x, indices=indices, scales=scales)
+    _dense(x=x, indices=indices, scales=scales)
     T, D = x.shape
     T_idx, K = indices.shape
     if T_idx != T:
-        raise ValueError(f"indices first dim {T_idx} must match x first dim {T}")
+        raise ValueError(f"indices cover {T_idx} tokens, x has {T}")
     if scales is not None:
-        if not scales.is_cuda:
-            raise ValueError("scales must be a CUDA tensor")
-        if not scales.is_contiguous():
-            raise ValueError("scales must be contiguous")
-        if scales.numel() != T * K:
-            raise ValueError(
-                f"scales must have T*K={T*K} elements, got {scales.numel()}. "
-                f"Expected shape [T={T}, K={K}] in ORIGINAL order (not sorted).")
+        _counted(scales, "scales", T * K, f" (one per (token, slot) pair in token order: [{T}, {K}])")
     if out is None:
         out = torch.empty((T * K, D), dtype=x.dtype, device=x.device)
     else:
-        if tuple(out.shape) != (T * K, D):
-            raise ValueError(f"out shape {tuple(out.shape)} must be [{T * K}, {D}]")
+        _shaped(out, "out", T * K, D)
         if out.dtype != x.dtype or out.stride(1) != 1:
             raise ValueError("out must have x's dtype and unit column stride")
     rc = lib().fx_moe_scatter(ptr(x), ptr(indices), _is64(indices), ptr(scales),
@@ -164,24 +161,16 @@ def flextrain_moe_scatter(x, indices, scales=None, out=None):
 
 def flextrain_moe_scatter_routing_weights(weights, indices, out=None):
     """``out[indices[i]] = weights[i]``; flextrain/ops/_kernels/moe.py:1053-1127."""
-    if not weights.is_cuda:
-        raise ValueError("weights must be a CUDA tensor")
-    if not indices.is_cuda:
-        raise ValueError("indices must be a CUDA tensor")
-    if weights.shape != indices.shape:
-        raise ValueError(f"weights shape {weights.shape} must match indices shape {indices.shape}")
+    _on_gpu(weights=weights, indices=indices)
+    _shaped(weights, "weights", *indices.shape)
     w_flat = weights.flatten()
     idx_flat = indices.flatten()
-    if not w_flat.is_contiguous():
-        raise ValueError("weights must be contiguous")
-    if not idx_flat.is_contiguous():
-        raise ValueError("indices must be contiguous")
+    _dense(weights=w_flat, indices=idx_flat)
     N = w_flat.numel()
     if out is None:
         out = torch.empty_like(w_flat)
     else:
-        if out.numel() != N:
-            raise ValueError(f"out must have {N} elements, got {out.numel()}")
+        _counted(out, "out", N)
         if out.dtype != w_flat.dtype or not out.is_contiguous():
             raise ValueError("out must be contiguous with the weights' dtype")
     rc = lib().fx_moe_scatter_weights(ptr(w_flat), ptr(idx_flat), _is64(idx_flat), ptr(out), N,
@@ -212,43 +201,23 @@ def flextrain_moe_row_sources(indices, out=None):
 def flextrain_moe_gather(expert_out, indices, weights=None, residual=None, out=None):
     """``out[t] = residual[t] + sum_k weights[t,k] * expert_out[indices[t,k]]``
     with an fp32 accumulator; flextrain/ops/_kernels/moe.py:1130-1271."""
-    if not expert_out.is_cuda:
-        raise ValueError("expert_out must be a CUDA tensor")
-    if not indices.is_cuda:
-        raise ValueError("indices must be a CUDA tensor")
-    if not expert_out.is_contiguous():
-        raise ValueError("expert_out must be contiguous")
-    if not indices.is_contiguous():
-        raise ValueError("indices must be contiguous")
+    _on_gpu(expert_out=expert_out, indices=indices, residual=residual, weights=weights)
+    _dense(expert_out=expert_out, indices=indices, residual=residual, weights=weights)
     T, K = indices.shape
-    _, D = expert_out.shape
-    if expert_out.shape[0] != T * K:
-        raise ValueError(
-            f"expert_out has {expert_out.shape[0]} rows but expected T*K={T * K} for T={T}, K={K}")
+    rows, D = expert_out.shape
+    if rows != T * K:
+        raise ValueError(f"expert_out has {rows} rows, the mapping routes {T} x {K} = {T * K}")
     if residual is not None:
-        if not residual.is_cuda:
-            raise ValueError("residual must be a CUDA tensor")
-        if not residual.is_contiguous():
-            raise ValueError("residual must be contiguous")
-        if tuple(residual.shape) != (T, D):
-            raise ValueError(f"residual shape {tuple(residual.shape)} must be [{T}, {D}]")
+        _shaped(residual, "residual", T, D)
     if weights is not None:
-        if not weights.is_cuda:
-            raise ValueError("weights must be a CUDA tensor")
-        if not weights.is_contiguous():
-            raise ValueError("weights must be contiguous")
-        if tuple(weights.shape) != (T, K):
-            raise ValueError(
-                f"weights shape {tuple(weights.shape)} must be [{T}, {K}] in ORIGINAL order. "
-                f"Do NOT pass router_weights_sorted here - use the original router_weights.")
+        # one weight per (token, slot) pair in TOKEN order, not the expert-sorted copy
+        _shaped(weights, "weights", T, K)
     if out is None:
         out_dtype = residual.dtype if residual is not None else expert_out.dtype
         out = torch.empty((T, D), dtype=out_dtype, device=expert_out.device)
     else:
-        if not out.is_contiguous():
-            raise ValueError("out must be contiguous")
-        if tuple(out.shape) != (T, D):
-            raise ValueError(f"out shape {tuple(out.shape)} must be [{T}, {D}]")
+        _dense(out=out)
+        _shaped(out, "out", T, D)
     rc = lib().fx_moe_gather(ptr(expert_out), ptr(indices), _is64(indices), ptr(weights),
                              dtype_enum(weights.dtype) if weights is not None else 0, ptr(residual),
                              dtype_enum(residual.dtype) if residual is not None else 0, ptr(out),
@@ -265,24 +234,19 @@ def _row_major(t, name):
 
 def flextrain_swiglu_moe_fwd(x, w=None, out=None):
     """``silu(x[:, F:]) * x[:, :F] (* w)``; flextrain/ops/_kernels/moe.py:1274-1320."""
-    if not x.is_cuda:
-        raise ValueError("x must be a CUDA tensor")
-    if w is not None and not w.is_cuda:
-        raise ValueError("w must be a CUDA tensor")
+    _on_gpu(x=x, w=w)
     T, F2 = x.shape
     if F2 % 2 != 0:
-        raise ValueError(f"x last dimension must be even (got {F2}), as it contains packed [value, gate]")
+        raise ValueError(f"x rows are packed [value | gate] halves; {F2} columns do not split")
     F = F2 // 2
     _row_major(x, "x")
     if out is None:
         out = torch.empty((T, F), device=x.device, dtype=x.dtype)
     else:
-        if tuple(out.shape) != (T, F):
-            raise ValueError(f"out shape {tuple(out.shape)} must be [{T}, {F}]")
+        _shaped(out, "out", T, F)
         _row_major(out, "out")
     if w is not None:
-        if w.numel() != T:
-            raise ValueError(f"w must have {T} elements, got {w.numel()}")
+        _counted(w, "w", T)
         w = w.reshape(-1)
         if not w.is_contiguous():
             w = w.contiguous()
@@ -294,29 +258,20 @@ def flextrain_swiglu_moe_fwd(x, w=None, out=None):
 
 
 def _swiglu_moe_bwd(dout, x, w, dx, dw, fwd_act, prescaled, dname):
-    if not dout.is_cuda:
-        raise ValueError(f"{dname} must be a CUDA tensor")
-    if not x.is_cuda:
-        raise ValueError("x must be a CUDA tensor")
-    if not w.is_cuda:
-        raise ValueError("w must be a CUDA tensor")
+    _on_gpu(**{dname: dout, "x": x, "w": w})
     T, F = dout.shape
-    if x.shape[0] != T:
-        raise ValueError(f"x first dim {x.shape[0]} must match {dname} first dim {T}")
-    if x.shape[1] != 2 * F:
-        raise ValueError(f"x second dim {x.shape[1]} must be 2*F={2*F}")
-    if w.numel() != T:
-        raise ValueError(f"w must have {T} elements, got {w.numel()}")
+    _shaped(x, "x", T, 2 * F)
+    _counted(w, "w", T)
     if dx is None:
         dx = torch.empty_like(x)
-    elif dx.shape != x.shape:
-        raise ValueError(f"dx shape {dx.shape} must match x shape {x.shape}")
+    else:
+        _shaped(dx, "dx", *x.shape)
     if dw is None:
         dw = torch.empty((T,), device=x.device, dtype=torch.float32)
-    elif dw.numel() != T:
-        raise ValueError(f"dw must have {T} elements, got {dw.numel()}")
-    if fwd_act is not None and tuple(fwd_act.shape) != (T, F):
-        raise ValueError(f"fwd_act shape {tuple(fwd_act.shape)} must be [{T}, {F}]")
+    else:
+        _counted(dw, "dw", T)
+    if fwd_act is not None:
+        _shaped(fwd_act, "fwd_act", T, F)
     for t, nm in ((dout, dname), (x, "x"), (dx, "dx"), (fwd_act, "fwd_act")):
         if t is not None:
             _row_major(t, nm)
@@ -350,40 +305,26 @@ def flextrain_moe_router_gate_bwd(probs, dprobs, indices, chosen_experts, dlogit
                                   mode="topk_then_softmax", logits=None):
     """Accumulate the router softmax Jacobian into ``dlogits``;
     flextrain/ops/_kernels/moe.py:1527-1655."""
-    if not probs.is_contiguous():
-        raise ValueError("probs must be contiguous")
-    if not dprobs.is_contiguous():
-        raise ValueError("dprobs must be contiguous")
-    if not indices.is_contiguous():
-        raise ValueError("indices must be contiguous")
-    if not chosen_experts.is_contiguous():
-        raise ValueError("chosen_experts must be contiguous")
+    _dense(probs=probs, dprobs=dprobs, indices=indices, chosen_experts=chosen_experts)
     T, K = probs.shape
-    if dprobs.numel() != T * K:
-        raise ValueError(f"dprobs must have T*K={T*K} elements, got {dprobs.numel()}")
-    if tuple(indices.shape) != (T, K):
-        raise ValueError(f"indices shape {tuple(indices.shape)} must be [{T}, {K}]")
-    if tuple(chosen_experts.shape) != (T, K):
-        raise ValueError(f"chosen_experts shape {tuple(chosen_experts.shape)} must be [{T}, {K}]")
+    _counted(dprobs, "dprobs", T * K)
+    _shaped(indices, "indices", T, K)
+    _shaped(chosen_experts, "chosen_experts", T, K)
     if dlogits is None:
         if num_experts is None:
-            raise ValueError("num_experts must be provided if dlogits is not passed")
+            raise ValueError("without dlogits the expert count must be given (num_experts)")
         dlogits = torch.zeros((T, num_experts), device=probs.device, dtype=probs.dtype)
     else:
         if dlogits.shape[0] != T:
-            raise ValueError(f"dlogits first dim {dlogits.shape[0]} must be T={T}")
-        if not dlogits.is_contiguous():
-            raise ValueError("dlogits must be contiguous")
+            raise ValueError(f"dlogits has {dlogits.shape[0]} rows for {T} tokens")
+        _dense(dlogits=dlogits)
     E = dlogits.shape[1]
     mode_id = _routing_mode_id(mode)
     if mode_id == _MODE_SOFTMAX_THEN_TOPK:
         if logits is None:
-            raise ValueError("softmax_then_topk backward requires ``logits`` (the original router "
-                             "logits, shape [T, E])")
-        if tuple(logits.shape) != (T, E):
-            raise ValueError(f"logits shape {tuple(logits.shape)} must be [{T}, {E}]")
-        if not logits.is_contiguous():
-            raise ValueError("logits must be contiguous")
+            raise ValueError("softmax_then_topk recomputes the full softmax: pass the router logits (T, E)")
+        _shaped(logits, "logits", T, E)
+        _dense(logits=logits)
         if logits.dtype != dlogits.dtype:
             raise TypeError("logits and dlogits must share a dtype")
     if probs.dtype != dlogits.dtype:
@@ -401,21 +342,16 @@ def flextrain_load_balance_bwd(logits, expert_counts, num_experts, top_k, alpha=
                                dlogits=None):
     """``dlogits += (alpha*E/tokens_per_step) * p * (f - <f,p>)``;
     flextrain/ops/_kernels/moe.py:1658-1745."""
-    if not logits.is_cuda:
-        raise ValueError("logits must be a CUDA tensor")
-    if not expert_counts.is_cuda:
-        raise ValueError("expert_counts must be a CUDA tensor")
+    _on_gpu(logits=logits, expert_counts=expert_counts)
     T, E = logits.shape
     if E != num_experts:
-        raise ValueError(f"logits has {E} experts but num_experts={num_experts}")
-    if expert_counts.numel() != E:
-        raise ValueError(f"expert_counts must have {E} elements, got {expert_counts.numel()}")
+        raise ValueError(f"logits have {E} columns for num_experts = {num_experts}")
+    _counted(expert_counts, "expert_counts", E)
     if dlogits is None:
         dlogits = torch.zeros_like(logits)
-    elif tuple(dlogits.shape) != (T, E):
-        raise ValueError(f"dlogits shape {tuple(dlogits.shape)} must be [{T}, {E}]")
-    if not logits.is_contiguous() or not dlogits.is_contiguous():
-        raise ValueError("logits and dlogits must be contiguous")
+    else:
+        _shaped(dlogits, "dlogits", T, E)
+    _dense(logits=logits, dlogits=dlogits)
     if tokens_per_step == 0:
         tokens_per_step = T
     scale = alpha * E / tokens_per_step
