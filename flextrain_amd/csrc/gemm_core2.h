@@ -68,7 +68,9 @@ FX_DEV void stage2_load(Staged2<ROWS, NT>& st, const OperandView<T>& op, int k0,
             int g = op.origin + r;
             g = g < op.ext ? g : op.ext - 1;
             const int k = k0 + c * 8;
-            st.v[i] = k < K ? ldg16(op.base + (int64_t)g * op.ld + k) : zero;
+            // gathered rows: the tail reads the same (clamped) source rows as the direct loads of the full steps
+            const int64_t row = op.row_map != nullptr ? (int64_t)min(max(op.row_map[g], 0), op.map_rows - 1) : (int64_t)g;
+            st.v[i] = k < K ? ldg16(op.base + row * op.ld + k) : zero;
         }
     } else {
         // blocks of 8(k) x 8(mn): ROWS blocks in all; a lane holds N k-rows of one block

@@ -424,7 +424,7 @@ def test_fused_dgrad_swiglu_bwd_equals_the_two_launches(dev, E, TK, d, F, dprob_
         _close_scaled(dw[a:b].reshape(-1), want_dw.reshape(-1), f"router-weight gradient of expert {e}")
 
 
-@pytest.mark.parametrize("T,E,K,d,F", [(1200, 4, 2, 192, 136), (8192, 128, 8, 2048, 768)])
+@pytest.mark.parametrize("T,E,K,d,F", [(1200, 4, 2, 192, 136), (1200, 4, 2, 200, 136), (8192, 128, 8, 2048, 768)])
 def test_backward_launches_gather_unsorted_rows_bit_for_bit(dev, T, E, K, d, F):
     """The expert backward without expert-sorted copies of dy and x: the fused dgrad launch (rows of
     the unsorted upstream gradient through the row map) and both weight-gradient launches (unsorted
