@@ -1,0 +1,134 @@
+// Host stand-in for <hip/hip_runtime.h>: the device code of this package's non-MFMA kernels compiled as
+// ordinary C++ and run on the CPU, one workgroup at a time, every GPU lane a cooperative fiber.
+//
+// What it is for: running the real kernel source (and the real host-side launch code: grid sizes, kernel
+// selection, workspace use) against buffers that end at inaccessible guard pages, so that an access one
+// element outside any operand kills the test, and comparing results with the CPU oracle.  Test
+// infrastructure only: nothing in the package includes it.
+//
+// Execution model: a launch runs its workgroups in order; a workgroup's lanes are fibers (ucontext) that
+// run until they meet a workgroup barrier, a wave-level exchange or their end.  __syncthreads() releases
+// when every lane still alive has arrived; wave operations exchange through one slot per lane.  Lanes
+// that returned count as arrived (on the GPU their wave either left the barrier's count or carries them
+// masked off).  __shared__ variables are statics: one workgroup exists at a time.
+#pragma once
+#include <ucontext.h>
+
+#include <algorithm>
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <functional>
+#include <vector>
+
+#define __global__
+#define __device__
+#define __host__
+#define __forceinline__ inline
+#define __launch_bounds__(...)
+#define __shared__ static
+#define __align__(n) __attribute__((aligned(n)))
+#define HIP_SYMBOL(x) (&(x))
+
+struct dim3 {
+    unsigned x, y, z;
+    dim3(unsigned a = 1, unsigned b = 1, unsigned c = 1) : x(a), y(b), z(c) {}
+};
+struct alignas(16) float4 { float x, y, z, w; };
+struct alignas(8) float2 { float x, y; };
+struct alignas(16) int4 { int x, y, z, w; };
+struct alignas(8) uint2 { unsigned x, y; };
+struct alignas(16) uint4 { unsigned x, y, z, w; };
+inline float4 make_float4(float x, float y, float z, float w) { return float4{x, y, z, w}; }
+inline float2 make_float2(float x, float y) { return float2{x, y}; }
+inline uint2 make_uint2(unsigned x, unsigned y) { return uint2{x, y}; }
+typedef void* hipStream_t;
+typedef int hipError_t;
+enum { hipSuccess = 0, hipErrorInvalidValue = 1 };
+enum { hipFuncAttributeMaxDynamicSharedMemorySize = 8, hipDeviceAttributeMultiprocessorCount = 63 };
+inline hipError_t hipGetLastError() { return hipSuccess; }
+inline const char* hipGetErrorString(hipError_t) { return "host simulation"; }
+inline hipError_t hipGetDevice(int* d) { *d = 0; return hipSuccess; }
+inline hipError_t hipDeviceGetAttribute(int* v, int, int) { *v = 256; return hipSuccess; }
+template <typename F> inline hipError_t hipFuncSetAttribute(F, int, int) { return hipSuccess; }
+template <typename T> inline hipError_t hipGetSymbolAddress(void** out, T* sym) { *out = (void*)sym; return hipSuccess; }
+
+namespace hostsim {
+
+struct Idx { unsigned x, y, z; };
+extern Idx g_thread, g_block;
+extern dim3 g_block_dim, g_grid_dim;
+extern unsigned char* g_dynamic_lds;
+
+void launch(dim3 grid, dim3 block, size_t lds_bytes, const std::function<void()>& body);
+void sync_threads();
+void sync_wave();
+unsigned lane_slot();                     // index of the running lane's exchange slot
+extern uint64_t g_exchange[];             // one 8-byte slot per lane of the workgroup
+extern unsigned char g_alive[];           // 1 while the lane has not returned
+unsigned flat_thread();
+
+template <typename T>
+inline T exchange(T v, int src_lane_in_wave) {
+    static_assert(sizeof(T) <= 8, "exchange slot");
+    const unsigned me = flat_thread();
+    const unsigned wave0 = me & ~63u;
+    uint64_t raw = 0;
+    memcpy(&raw, &v, sizeof(T));
+    g_exchange[me] = raw;
+    sync_wave();
+    T out = v;
+    const unsigned src = wave0 + (unsigned)src_lane_in_wave;
+    if (src_lane_in_wave >= 0 && src_lane_in_wave < 64 && src < g_block_dim.x * g_block_dim.y * g_block_dim.z && g_alive[src])
+        memcpy(&out, &g_exchange[src], sizeof(T));
+    sync_wave();
+    return out;
+}
+
+}  // namespace hostsim
+
+#define threadIdx hostsim::g_thread
+#define blockIdx hostsim::g_block
+#define blockDim hostsim::g_block_dim
+#define gridDim hostsim::g_grid_dim
+
+inline void __syncthreads() { hostsim::sync_threads(); }
+template <typename T> inline T __shfl_xor(T v, int mask, int width = 64) { (void)width; return hostsim::exchange(v, (int)((hostsim::flat_thread() & 63u) ^ (unsigned)mask)); }
+template <typename T> inline T __shfl_up(T v, unsigned delta, int width = 64) {
+    (void)width;
+    const int lane = (int)(hostsim::flat_thread() & 63u);
+    return hostsim::exchange(v, lane - (int)delta >= 0 ? lane - (int)delta : lane);
+}
+template <typename T> inline T __shfl_down(T v, unsigned delta, int width = 64) {
+    (void)width;
+    const int lane = (int)(hostsim::flat_thread() & 63u);
+    return hostsim::exchange(v, lane + (int)delta < 64 ? lane + (int)delta : lane);
+}
+template <typename T> inline T __shfl(T v, int src, int width = 64) { (void)width; return hostsim::exchange(v, src); }
+inline int __any(int pred) {
+    const unsigned me = hostsim::flat_thread(), wave0 = me & ~63u;
+    const unsigned lanes = hostsim::g_block_dim.x * hostsim::g_block_dim.y * hostsim::g_block_dim.z;
+    hostsim::g_exchange[me] = pred != 0;
+    hostsim::sync_wave();
+    int any = 0;
+    for (unsigned l = wave0; l < wave0 + 64 && l < lanes; ++l) any |= hostsim::g_alive[l] && hostsim::g_exchange[l] != 0;
+    hostsim::sync_wave();
+    return any;
+}
+template <typename T> inline T atomicAdd(T* p, T v) { T old = *p; *p = old + v; return old; }      // fibers never preempt each other
+template <typename T> inline T atomicOr(T* p, T v) { T old = *p; *p = old | v; return old; }
+template <typename T> inline T atomicMax(T* p, T v) { T old = *p; *p = std::max(old, v); return old; }
+
+// gfx950 builtins the kernels use, by their documented meaning
+#define __builtin_amdgcn_rcpf(x) (1.0f / (x))
+#define __builtin_amdgcn_exp2f(x) exp2f(x)
+#define __builtin_amdgcn_readfirstlane(x) (x)          /* only ever applied to wave-uniform values */
+#define __builtin_amdgcn_wave_barrier() hostsim::sync_wave()
+#define __builtin_amdgcn_fence(...) ((void)0)
+#define __builtin_amdgcn_sched_barrier(x) ((void)0)
+#define __builtin_amdgcn_s_setprio(x) ((void)0)
+inline float rsqrtf(float x) { return 1.0f / sqrtf(x); }
+#define __expf(x) expf(x)
+#define __logf(x) logf(x)

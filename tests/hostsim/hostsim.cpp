@@ -1,0 +1,115 @@
+// Runtime of the host simulation (see hip/hip_runtime.h in this directory): workgroups in order, lanes as fibers.
+#include <sys/mman.h>
+
+#include "hip/hip_runtime.h"
+
+namespace hostsim {
+
+Idx g_thread, g_block;
+dim3 g_block_dim, g_grid_dim;
+constexpr int MAX_LANES = 1024;
+constexpr size_t STACK_BYTES = 256 * 1024;
+uint64_t g_exchange[MAX_LANES];
+unsigned char g_alive[MAX_LANES];
+alignas(256) static unsigned char g_lds_store[160 * 1024];
+unsigned char* g_dynamic_lds = g_lds_store;
+
+static ucontext_t g_scheduler, g_lane_ctx[MAX_LANES];
+static char* g_stacks = nullptr;
+static Idx g_lane_idx[MAX_LANES];
+static int g_current = 0, g_lanes = 0;
+static const std::function<void()>* g_body = nullptr;
+static unsigned g_alive_block = 0, g_arrived_block = 0, g_generation_block = 0;
+static unsigned g_alive_wave[MAX_LANES / 64], g_arrived_wave[MAX_LANES / 64], g_generation_wave[MAX_LANES / 64];
+static unsigned long g_progress = 0;
+
+unsigned flat_thread() { return (unsigned)g_current; }
+
+static void yield() { swapcontext(&g_lane_ctx[g_current], &g_scheduler); }
+
+void sync_threads() {
+    const unsigned gen = g_generation_block;
+    if (++g_arrived_block >= g_alive_block) {
+        g_arrived_block = 0;
+        ++g_generation_block;
+        ++g_progress;
+        return;
+    }
+    while (g_generation_block == gen) yield();
+}
+
+void sync_wave() {
+    const int w = g_current >> 6;
+    const unsigned gen = g_generation_wave[w];
+    if (++g_arrived_wave[w] >= g_alive_wave[w]) {
+        g_arrived_wave[w] = 0;
+        ++g_generation_wave[w];
+        ++g_progress;
+        return;
+    }
+    while (g_generation_wave[w] == gen) yield();
+}
+
+static void lane_main() {
+    (*g_body)();
+    // a lane that returns no longer takes part in barriers; one that was the last awaited releases them
+    const int w = g_current >> 6;
+    g_alive[g_current] = 0;
+    ++g_progress;
+    if (--g_alive_block > 0 && g_arrived_block >= g_alive_block) { g_arrived_block = 0; ++g_generation_block; }
+    if (--g_alive_wave[w] > 0 && g_arrived_wave[w] >= g_alive_wave[w]) { g_arrived_wave[w] = 0; ++g_generation_wave[w]; }
+    swapcontext(&g_lane_ctx[g_current], &g_scheduler);
+}
+
+void launch(dim3 grid, dim3 block, size_t lds_bytes, const std::function<void()>& body) {
+    const int lanes = (int)(block.x * block.y * block.z);
+    if (lanes <= 0 || lanes > MAX_LANES) { fprintf(stderr, "hostsim: workgroup of %d lanes\n", lanes); abort(); }
+    if (lds_bytes > sizeof(g_lds_store)) { fprintf(stderr, "hostsim: %zu bytes of dynamic LDS\n", lds_bytes); abort(); }
+    if ((uint64_t)grid.x * grid.y * grid.z == 0) { fprintf(stderr, "hostsim: empty grid\n"); abort(); }
+    if (!g_stacks) {
+        g_stacks = (char*)mmap(nullptr, STACK_BYTES * MAX_LANES, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0);
+        if (g_stacks == (char*)MAP_FAILED) { perror("hostsim: mmap"); abort(); }
+    }
+    g_body = &body;
+    g_block_dim = block;
+    g_grid_dim = grid;
+    g_lanes = lanes;
+    for (unsigned bz = 0; bz < grid.z; ++bz)
+        for (unsigned by = 0; by < grid.y; ++by)
+            for (unsigned bx = 0; bx < grid.x; ++bx) {
+                g_block = Idx{bx, by, bz};
+                g_alive_block = (unsigned)lanes;
+                g_arrived_block = 0;
+                for (int w = 0; w < MAX_LANES / 64; ++w) { g_alive_wave[w] = 0; g_arrived_wave[w] = 0; }
+                for (int i = 0; i < lanes; ++i) {
+                    g_lane_idx[i] = Idx{(unsigned)i % block.x, ((unsigned)i / block.x) % block.y, (unsigned)i / (block.x * block.y)};
+                    g_alive[i] = 1;
+                    ++g_alive_wave[i >> 6];
+                    getcontext(&g_lane_ctx[i]);
+                    g_lane_ctx[i].uc_stack.ss_sp = g_stacks + (size_t)i * STACK_BYTES;
+                    g_lane_ctx[i].uc_stack.ss_size = STACK_BYTES;
+                    g_lane_ctx[i].uc_link = nullptr;
+                    makecontext(&g_lane_ctx[i], lane_main, 0);
+                }
+                unsigned left = (unsigned)lanes;
+                while (left > 0) {
+                    const unsigned long before = g_progress;
+                    left = 0;
+                    for (int i = 0; i < lanes; ++i) {
+                        if (!g_alive[i]) continue;
+                        g_current = i;
+                        g_thread = g_lane_idx[i];
+                        swapcontext(&g_scheduler, &g_lane_ctx[i]);
+                        left += g_alive[i];
+                    }
+                    if (left > 0 && g_progress == before) {
+                        fprintf(stderr, "hostsim: workgroup (%u,%u,%u) is stuck: %u lanes wait at a barrier that the others never reach\n",
+                                bx, by, bz, left);
+                        abort();
+                    }
+                }
+            }
+    g_body = nullptr;
+}
+
+}  // namespace hostsim

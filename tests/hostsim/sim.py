@@ -1,0 +1,64 @@
+"""Python side of the host simulation: the simulated library bound with the package's own ctypes
+signatures, and tensors whose storage ends at an inaccessible page."""
+from __future__ import annotations
+
+import ctypes
+import mmap
+import os
+
+import torch
+
+from . import build as _build
+
+_PAGE = mmap.PAGESIZE
+_libc = ctypes.CDLL(None, use_errno=True)
+_libc.mprotect.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+_keep = []          # the mappings live as long as the process: tensors made from them hold no reference
+_lib = None
+
+
+def lib():
+    """The simulated libflexhip, every entry point it exports bound with the signature the package binds
+    the real library with (``flextrain_amd._lib._SIGNATURES``)."""
+    global _lib
+    if _lib is None:
+        from flextrain_amd._lib import _SIGNATURES
+
+        handle = ctypes.CDLL(_build.build())
+        for name, (restype, argtypes) in _SIGNATURES.items():
+            fn = getattr(handle, name, None)
+            if fn is not None:
+                fn.restype, fn.argtypes = restype, argtypes
+        _lib = handle
+    return _lib
+
+
+def guard(t: torch.Tensor, align: int = 16) -> torch.Tensor:
+    """A copy of ``t`` (contiguous) whose last byte is followed, within ``align`` bytes, by a page that
+    may be neither read nor written; the page before the mapping's first is protected too."""
+    t = t.detach().contiguous()
+    nbytes = t.numel() * t.element_size()
+    body = (max(nbytes, 1) + _PAGE - 1) // _PAGE * _PAGE
+    mm = mmap.mmap(-1, body + 2 * _PAGE)
+    base = ctypes.addressof(ctypes.c_char.from_buffer(mm))
+    if _libc.mprotect(base, _PAGE, 0) != 0 or _libc.mprotect(base + _PAGE + body, _PAGE, 0) != 0:
+        raise OSError(ctypes.get_errno(), "mprotect")
+    start = (_PAGE + body - nbytes) // align * align
+    _keep.append(mm)
+    if nbytes == 0:
+        return torch.empty_like(t)
+    out = torch.frombuffer(mm, dtype=t.dtype, count=t.numel(), offset=start).view(t.shape)
+    out.copy_(t)
+    return out
+
+
+def p(t):
+    return None if t is None else t.data_ptr()
+
+
+DT = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+
+
+def pi64(t):
+    """An int64 tensor as the POINTER(c_int64) the stride arguments are declared with."""
+    return None if t is None else ctypes.cast(t.data_ptr(), ctypes.POINTER(ctypes.c_int64))
