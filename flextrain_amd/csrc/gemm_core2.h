@@ -482,6 +482,7 @@ FX_DEV void epilogue_tile(f32x16_t (&acc)[WM / 32][WN / 32], const TD* C, TD* D,
     const bool pre_c = vec_ok && beta != 0.f;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
+        // lockstep: every lane of the wave has read the previous band back before this one is staged
         if (pre_c && i % CB == 0) {
 #pragma unroll
             for (int b = 0; b < CB; ++b)
@@ -506,7 +507,7 @@ FX_DEV void epilogue_tile(f32x16_t (&acc)[WM / 32][WN / 32], const TD* C, TD* D,
                 *reinterpret_cast<f32x4_t*>(stage + (lane & 31) * PITCH + j * 32 + 8 * g + 4 * (lane >> 5)) = q;
             }
         if (LOADS_LAND && i == TM - 1) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        // a wave reads back only what it wrote itself; its LDS accesses complete in order
+        // lockstep: a wave reads back only what it wrote itself; its LDS accesses complete in order
 #pragma unroll
         for (int t = 0; t < PER_LANE; ++t) {
             const int id = t * 64 + lane;
@@ -757,6 +758,7 @@ FX_DEV void gemm_tile2_glu(const OperandView<T>& A, const OperandView<T>& B, T* 
     const int row_base = A.origin + wm * WM, col_base = B.origin + wn * HC;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
+        // lockstep: every lane of the wave has read the previous band back before this one is staged
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
             T* dst = (j < TN / 2 ? st1 : st2) + (lane & 31) * PITCH + (j % (TN / 2)) * 32 + 4 * (lane >> 5);
@@ -766,7 +768,7 @@ FX_DEV void gemm_tile2_glu(const OperandView<T>& A, const OperandView<T>& B, T* 
                 *reinterpret_cast<t4_t*>(dst + 8 * g) = q;
             }
         }
-        // a wave reads back only what it wrote itself; its LDS accesses complete in order
+        // lockstep: a wave reads back only what it wrote itself; its LDS accesses complete in order
 #pragma unroll
         for (int t = 0; t < PER_LANE; ++t) {
             const int id = t * 64 + lane;

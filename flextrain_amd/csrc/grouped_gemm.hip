@@ -284,6 +284,7 @@ FX_DEV void epilogue_swiglu_bwd(f32x16_t (&acc)[WM / 32][WN / 32], const T* __re
     };
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
+        // lockstep: every lane of the wave has read the previous band back before this one is staged
         request(i, 0);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -294,7 +295,7 @@ FX_DEV void epilogue_swiglu_bwd(f32x16_t (&acc)[WM / 32][WN / 32], const T* __re
                 *reinterpret_cast<f32x4_t*>(stage + (lane & 31) * PITCH + j * 32 + 8 * g + 4 * (lane >> 5)) = q;
             }
         if (LOADS_LAND && i == TM - 1) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        // a wave reads back only what it wrote itself; its LDS accesses complete in order
+        // lockstep: a wave reads back only what it wrote itself; its LDS accesses complete in order
 #pragma unroll
         for (int t = 0; t < PER_LANE; ++t) {
             const int id = t * 64 + lane;

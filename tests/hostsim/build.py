@@ -18,7 +18,9 @@ CSRC = os.path.join(ROOT, "flextrain_amd", "csrc")
 OUT = os.path.join(HERE, "_build")
 LIB = os.path.join(OUT, "libflexhip_hostsim.so")
 CLANG = "/opt/rocm/lib/llvm/bin/clang++"
-SOURCES = ("rmsnorm.hip", "rope.hip", "glu.hip", "softmax_ce.hip", "adamw.hip", "moe_route.hip", "moe_data.hip", "embed.hip")
+SOURCES = ("rmsnorm.hip", "rope.hip", "glu.hip", "softmax_ce.hip", "adamw.hip", "moe_route.hip", "moe_data.hip", "embed.hip",
+           "gemm.hip", "gemm_glu.hip", "gemm_ksum.hip", "gemm_segments.hip", "grouped_gemm.hip")
+HEADERS = ("common.h", "gemm_core.h", "gemm_core2.h")
 
 
 def _match_forward(text, i, open_ch, close_ch):
@@ -84,24 +86,48 @@ def rewrite_launches(text):
 
 
 def rewrite_dynamic_lds(text):
-    return re.sub(r"extern\s+__shared__\s+(?:__align__\(\d+\)\s+)?([A-Za-z_0-9:]+)\s+(\w+)\[\];",
+    return re.sub(r"extern\s+__shared__\s+(?:__align__\(\d+\)\s+)?([A-Za-z_0-9: ]+?)\s+(\w+)\[\];",
                   r"\1* \2 = reinterpret_cast<\1*>(hostsim::g_dynamic_lds);", text)
+
+
+def rewrite_asm(text):
+    """The three kinds of inline assembly in the GEMM code: the two LDS-DMA loads become calls of the
+    stand-in, the wait-count instructions (the stand-in load completes at once) become nothing."""
+    def one(m):
+        body = m.group(1)
+        if "global_load_lds_dwordx4 %1, off" in body:
+            return "hostsim::lds_dma16(lds_addr, gptr);"
+        if "global_load_lds_dwordx4 %1, %2" in body:
+            return "hostsim::lds_dma16(lds_addr, reinterpret_cast<const char*>(sbase) + lane_off);"
+        assert "s_waitcnt" in body, f"inline assembly the host simulation has no stand-in for: {body[:80]}"
+        return "((void)0);"
+    return re.sub(r"asm volatile\((.*?)\);", one, text)
+
+
+def rewrite_lockstep(text):
+    """A GPU wave runs its lanes in lockstep, so a wave may stage values in LDS and read its neighbours'
+    values back with no barrier in between; fibers do not.  The sources mark those points with comment lines
+    that start with ``// lockstep:``; here each becomes a wave-level rendezvous."""
+    return re.sub(r"^(\s*)// lockstep:", r"\1hostsim::sync_wave();  // lockstep:", text, flags=re.M)
 
 
 def build(force=False):
     os.makedirs(OUT, exist_ok=True)
-    inputs = [os.path.join(CSRC, f) for f in SOURCES] + [os.path.join(CSRC, "common.h"), os.path.join(HERE, "hostsim.cpp"),
-                                                            os.path.join(HERE, "hip", "hip_runtime.h"), os.path.abspath(__file__)]
+    inputs = [os.path.join(CSRC, f) for f in SOURCES + HEADERS] + [os.path.join(HERE, "hostsim.cpp"),
+                                                                      os.path.join(HERE, "hip", "hip_runtime.h"), os.path.abspath(__file__)]
     if not force and os.path.exists(LIB) and all(os.path.getmtime(LIB) >= os.path.getmtime(p) for p in inputs):
         return LIB
     objects = []
+    for name in HEADERS:                 # the headers with inline assembly are rewritten too and found first
+        with open(os.path.join(OUT, name), "w") as f:
+            f.write(rewrite_lockstep(rewrite_asm(open(os.path.join(CSRC, name)).read())))
     for name in SOURCES:
         text = open(os.path.join(CSRC, name)).read()
         cpp = os.path.join(OUT, name.replace(".hip", "_hostsim.cpp"))
         with open(cpp, "w") as f:
-            f.write(rewrite_dynamic_lds(rewrite_launches(text)))
+            f.write(rewrite_lockstep(rewrite_asm(rewrite_dynamic_lds(rewrite_launches(text)))))
         objects.append(cpp)
-    cmd = [CLANG, "-std=c++17", "-O1", "-g", "-fPIC", "-shared", "-D__HIP__", "-Wno-everything", "-I", HERE, "-I", CSRC,
+    cmd = [CLANG, "-std=c++17", "-O1", "-g", "-fPIC", "-shared", "-D__HIP__", "-Wno-everything", "-I", HERE, "-I", OUT, "-I", CSRC,
            "-I", os.path.join(ROOT, "include"), "-o", LIB, os.path.join(HERE, "hostsim.cpp")] + objects
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:

@@ -32,6 +32,9 @@
 #define __align__(n) __attribute__((aligned(n)))
 #define HIP_SYMBOL(x) (&(x))
 
+using std::max;
+using std::min;
+
 struct dim3 {
     unsigned x, y, z;
     dim3(unsigned a = 1, unsigned b = 1, unsigned c = 1) : x(a), y(b), z(c) {}
@@ -120,6 +123,70 @@ inline int __any(int pred) {
 template <typename T> inline T atomicAdd(T* p, T v) { T old = *p; *p = old + v; return old; }      // fibers never preempt each other
 template <typename T> inline T atomicOr(T* p, T v) { T old = *p; *p = old | v; return old; }
 template <typename T> inline T atomicMax(T* p, T v) { T old = *p; *p = std::max(old, v); return old; }
+
+namespace hostsim {
+extern unsigned char (*g_wave_buf)[64][32];     // [wave][lane][32 bytes]: operands published for a wave-wide instruction
+
+// global_load_lds_dwordx4: lane l of the wave copies 16 bytes from its global address to lds_addr + 16 l.
+// Completes at once (one of the orders the hardware may take; the kernels wait before they read).
+inline void lds_dma16(unsigned lds_addr, const void* gptr) {
+    memcpy(reinterpret_cast<void*>((uintptr_t)lds_addr + 16u * (flat_thread() & 63u)), gptr, 16);
+}
+
+// v_mfma_f32_32x32x16 (bf16 / f16): D = A (32 x 16) * B (16 x 32) + C.  Lane l supplies A[l % 32][8 (l / 32) .. + 7]
+// and B[8 (l / 32) .. + 7][l % 32]; register v of lane l is D[8 (v / 4) + 4 (l / 32) + v % 4][l % 32].
+template <typename Frag, typename Acc>
+inline Acc mfma32x32x16(Frag a, Frag b, Acc c) {
+    const unsigned me = flat_thread(), w = me >> 6, l = me & 63u;
+    memcpy(&g_wave_buf[w][l][0], &a, 16);
+    memcpy(&g_wave_buf[w][l][16], &b, 16);
+    sync_wave();
+    typedef decltype(a[0] + a[0]) dummy_t;
+    (void)sizeof(dummy_t);
+    for (int v = 0; v < 16; ++v) {
+        const unsigned row = 8u * (v / 4) + 4u * (l / 32) + (unsigned)(v % 4), col = l % 32;
+        float sum = c[v];
+        for (int k = 0; k < 16; ++k) {
+            Frag fa, fb;
+            memcpy(&fa, &g_wave_buf[w][row + 32u * (k / 8)][0], 16);
+            memcpy(&fb, &g_wave_buf[w][col + 32u * (k / 8)][16], 16);
+            sum += (float)fa[k % 8] * (float)fb[k % 8];
+        }
+        c[v] = sum;
+    }
+    sync_wave();
+    return c;
+}
+
+// ds_read_b64_tr_b16: inside each group of 16 lanes, lane s receives, for j = 0 .. 3, element s % 4 of the
+// 8 bytes that lane 4 j + s / 4 of the group addressed.
+template <typename V4>
+inline V4 ds_read_tr16(const void* addr) {
+    const unsigned me = flat_thread(), group0 = me & ~15u, s = me & 15u;
+    g_exchange[me] = (uint64_t)(uintptr_t)addr;
+    sync_wave();
+    V4 out;
+    for (unsigned j = 0; j < 4; ++j) {
+        const short* src = reinterpret_cast<const short*>((uintptr_t)g_exchange[group0 + 4 * j + s / 4]);
+        out[j] = src[s % 4];
+    }
+    sync_wave();
+    return out;
+}
+
+// v_perm_b32: byte i of the result is byte sel[i] of the 8 bytes {hi : lo} (0-3 from lo, 4-7 from hi).
+inline unsigned perm_b32(unsigned hi, unsigned lo, unsigned sel) {
+    const uint64_t both = ((uint64_t)hi << 32) | lo;
+    unsigned out = 0;
+    for (int i = 0; i < 4; ++i) out |= (unsigned)((both >> (8 * ((sel >> (8 * i)) & 7))) & 0xff) << (8 * i);
+    return out;
+}
+}  // namespace hostsim
+
+#define __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, x, y, z) hostsim::mfma32x32x16(a, b, c)
+#define __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, x, y, z) hostsim::mfma32x32x16(a, b, c)
+#define __builtin_amdgcn_ds_read_tr16_b64_v4i16(p) hostsim::ds_read_tr16<short __attribute__((ext_vector_type(4)))>((const void*)(p))
+#define __builtin_amdgcn_perm(hi, lo, sel) hostsim::perm_b32(hi, lo, sel)
 
 // gfx950 builtins the kernels use, by their documented meaning
 #define __builtin_amdgcn_rcpf(x) (1.0f / (x))

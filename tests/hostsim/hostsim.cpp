@@ -11,8 +11,21 @@ constexpr int MAX_LANES = 1024;
 constexpr size_t STACK_BYTES = 256 * 1024;
 uint64_t g_exchange[MAX_LANES];
 unsigned char g_alive[MAX_LANES];
-alignas(256) static unsigned char g_lds_store[160 * 1024];
-unsigned char* g_dynamic_lds = g_lds_store;
+// The LDS lives below 4 GB: the kernels keep LDS addresses as 32-bit values (as the hardware does) and the
+// stand-in for the LDS-DMA load turns them back into pointers.
+constexpr size_t LDS_BYTES = 160 * 1024;
+static unsigned char* map_lds() {
+    for (uintptr_t at = 0x40000000u; at < 0xF0000000u; at += 0x10000000u) {
+        void* p = mmap((void*)at, LDS_BYTES, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_FIXED_NOREPLACE, -1, 0);
+        if (p == (void*)at) return (unsigned char*)p;
+        if (p != MAP_FAILED) munmap(p, LDS_BYTES);
+    }
+    fprintf(stderr, "hostsim: no room below 4 GB for the LDS\n");
+    abort();
+}
+unsigned char* g_dynamic_lds = map_lds();
+static unsigned char g_wave_store[MAX_LANES / 64][64][32];
+unsigned char (*g_wave_buf)[64][32] = g_wave_store;
 
 static ucontext_t g_scheduler, g_lane_ctx[MAX_LANES];
 static char* g_stacks = nullptr;
@@ -64,7 +77,7 @@ static void lane_main() {
 void launch(dim3 grid, dim3 block, size_t lds_bytes, const std::function<void()>& body) {
     const int lanes = (int)(block.x * block.y * block.z);
     if (lanes <= 0 || lanes > MAX_LANES) { fprintf(stderr, "hostsim: workgroup of %d lanes\n", lanes); abort(); }
-    if (lds_bytes > sizeof(g_lds_store)) { fprintf(stderr, "hostsim: %zu bytes of dynamic LDS\n", lds_bytes); abort(); }
+    if (lds_bytes > LDS_BYTES) { fprintf(stderr, "hostsim: %zu bytes of dynamic LDS\n", lds_bytes); abort(); }
     if ((uint64_t)grid.x * grid.y * grid.z == 0) { fprintf(stderr, "hostsim: empty grid\n"); abort(); }
     if (!g_stacks) {
         g_stacks = (char*)mmap(nullptr, STACK_BYTES * MAX_LANES, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0);
