@@ -127,7 +127,7 @@ def build(force=False):
         with open(cpp, "w") as f:
             f.write(rewrite_lockstep(rewrite_asm(rewrite_dynamic_lds(rewrite_launches(text)))))
         objects.append(cpp)
-    cmd = [CLANG, "-std=c++17", "-O1", "-g", "-fPIC", "-shared", "-D__HIP__", "-Wno-everything", "-I", HERE, "-I", OUT, "-I", CSRC,
+    cmd = [CLANG, "-std=c++17", "-O2", "-g", "-fPIC", "-shared", "-D__HIP__", "-Wno-everything", "-I", HERE, "-I", OUT, "-I", CSRC,
            "-I", os.path.join(ROOT, "include"), "-o", LIB, os.path.join(HERE, "hostsim.cpp")] + objects
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:

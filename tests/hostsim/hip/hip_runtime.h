@@ -6,14 +6,12 @@
 // element outside any operand kills the test, and comparing results with the CPU oracle.  Test
 // infrastructure only: nothing in the package includes it.
 //
-// Execution model: a launch runs its workgroups in order; a workgroup's lanes are fibers (ucontext) that
+// Execution model: a launch runs its workgroups in order; a workgroup's lanes are fibers that
 // run until they meet a workgroup barrier, a wave-level exchange or their end.  __syncthreads() releases
 // when every lane still alive has arrived; wave operations exchange through one slot per lane.  Lanes
 // that returned count as arrived (on the GPU their wave either left the barrier's count or carries them
 // masked off).  __shared__ variables are statics: one workgroup exists at a time.
 #pragma once
-#include <ucontext.h>
-
 #include <algorithm>
 #include <cmath>
 #include <cstdint>
@@ -125,7 +123,7 @@ template <typename T> inline T atomicOr(T* p, T v) { T old = *p; *p = old | v; r
 template <typename T> inline T atomicMax(T* p, T v) { T old = *p; *p = std::max(old, v); return old; }
 
 namespace hostsim {
-extern unsigned char (*g_wave_buf)[64][32];     // [wave][lane][32 bytes]: operands published for a wave-wide instruction
+extern float (*g_wave_f32)[64][16];             // [wave][lane][8 of A, 8 of B]: operands published for a matrix instruction
 
 // global_load_lds_dwordx4: lane l of the wave copies 16 bytes from its global address to lds_addr + 16 l.
 // Completes at once (one of the orders the hardware may take; the kernels wait before they read).
@@ -138,20 +136,18 @@ inline void lds_dma16(unsigned lds_addr, const void* gptr) {
 template <typename Frag, typename Acc>
 inline Acc mfma32x32x16(Frag a, Frag b, Acc c) {
     const unsigned me = flat_thread(), w = me >> 6, l = me & 63u;
-    memcpy(&g_wave_buf[w][l][0], &a, 16);
-    memcpy(&g_wave_buf[w][l][16], &b, 16);
+    float* mine = g_wave_f32[w][l];
+    for (int j = 0; j < 8; ++j) { mine[j] = (float)a[j]; mine[8 + j] = (float)b[j]; }
     sync_wave();
-    typedef decltype(a[0] + a[0]) dummy_t;
-    (void)sizeof(dummy_t);
+    const float* b_lo = g_wave_f32[w][l % 32] + 8;            // B[0 .. 7][col], B[8 .. 15][col]
+    const float* b_hi = g_wave_f32[w][l % 32 + 32] + 8;
     for (int v = 0; v < 16; ++v) {
-        const unsigned row = 8u * (v / 4) + 4u * (l / 32) + (unsigned)(v % 4), col = l % 32;
+        const unsigned row = 8u * (v / 4) + 4u * (l / 32) + (unsigned)(v % 4);
+        const float* a_lo = g_wave_f32[w][row];
+        const float* a_hi = g_wave_f32[w][row + 32];
         float sum = c[v];
-        for (int k = 0; k < 16; ++k) {
-            Frag fa, fb;
-            memcpy(&fa, &g_wave_buf[w][row + 32u * (k / 8)][0], 16);
-            memcpy(&fb, &g_wave_buf[w][col + 32u * (k / 8)][16], 16);
-            sum += (float)fa[k % 8] * (float)fb[k % 8];
-        }
+        for (int k = 0; k < 8; ++k) sum += a_lo[k] * b_lo[k];
+        for (int k = 0; k < 8; ++k) sum += a_hi[k] * b_hi[k];
         c[v] = sum;
     }
     sync_wave();

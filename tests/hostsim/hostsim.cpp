@@ -24,10 +24,36 @@ static unsigned char* map_lds() {
     abort();
 }
 unsigned char* g_dynamic_lds = map_lds();
-static unsigned char g_wave_store[MAX_LANES / 64][64][32];
-unsigned char (*g_wave_buf)[64][32] = g_wave_store;
+static float g_wave_store[MAX_LANES / 64][64][16];
+float (*g_wave_f32)[64][16] = g_wave_store;
 
-static ucontext_t g_scheduler, g_lane_ctx[MAX_LANES];
+// Fiber switch: the callee-saved registers go on the old stack, the stack pointers are exchanged
+// (swapcontext would make a signal-mask system call per switch, and a GEMM tile makes millions).
+extern "C" void hostsim_switch(void** save_sp, void* load_sp);
+asm(R"(
+    .text
+    .globl hostsim_switch
+    .type hostsim_switch,@function
+hostsim_switch:
+    pushq %rbp
+    pushq %rbx
+    pushq %r12
+    pushq %r13
+    pushq %r14
+    pushq %r15
+    movq %rsp, (%rdi)
+    movq %rsi, %rsp
+    popq %r15
+    popq %r14
+    popq %r13
+    popq %r12
+    popq %rbx
+    popq %rbp
+    ret
+    .size hostsim_switch, .-hostsim_switch
+)");
+static void* g_scheduler_sp = nullptr;
+static void* g_lane_sp[MAX_LANES];
 static char* g_stacks = nullptr;
 static Idx g_lane_idx[MAX_LANES];
 static int g_current = 0, g_lanes = 0;
@@ -38,7 +64,7 @@ static unsigned long g_progress = 0;
 
 unsigned flat_thread() { return (unsigned)g_current; }
 
-static void yield() { swapcontext(&g_lane_ctx[g_current], &g_scheduler); }
+static void yield() { hostsim_switch(&g_lane_sp[g_current], g_scheduler_sp); }
 
 void sync_threads() {
     const unsigned gen = g_generation_block;
@@ -71,7 +97,8 @@ static void lane_main() {
     ++g_progress;
     if (--g_alive_block > 0 && g_arrived_block >= g_alive_block) { g_arrived_block = 0; ++g_generation_block; }
     if (--g_alive_wave[w] > 0 && g_arrived_wave[w] >= g_alive_wave[w]) { g_arrived_wave[w] = 0; ++g_generation_wave[w]; }
-    swapcontext(&g_lane_ctx[g_current], &g_scheduler);
+    hostsim_switch(&g_lane_sp[g_current], g_scheduler_sp);
+    abort();        // a finished lane is never resumed
 }
 
 void launch(dim3 grid, dim3 block, size_t lds_bytes, const std::function<void()>& body) {
@@ -98,11 +125,13 @@ void launch(dim3 grid, dim3 block, size_t lds_bytes, const std::function<void()>
                     g_lane_idx[i] = Idx{(unsigned)i % block.x, ((unsigned)i / block.x) % block.y, (unsigned)i / (block.x * block.y)};
                     g_alive[i] = 1;
                     ++g_alive_wave[i >> 6];
-                    getcontext(&g_lane_ctx[i]);
-                    g_lane_ctx[i].uc_stack.ss_sp = g_stacks + (size_t)i * STACK_BYTES;
-                    g_lane_ctx[i].uc_stack.ss_size = STACK_BYTES;
-                    g_lane_ctx[i].uc_link = nullptr;
-                    makecontext(&g_lane_ctx[i], lane_main, 0);
+                    // a fresh stack that hostsim_switch can "return" into: six saved registers, then lane_main as the
+                    // return address, at the alignment a called function expects
+                    void** top = reinterpret_cast<void**>(g_stacks + (size_t)(i + 1) * STACK_BYTES);
+                    *--top = nullptr;
+                    *--top = reinterpret_cast<void*>(&lane_main);
+                    for (int r = 0; r < 6; ++r) *--top = nullptr;
+                    g_lane_sp[i] = top;
                 }
                 unsigned left = (unsigned)lanes;
                 while (left > 0) {
@@ -112,7 +141,7 @@ void launch(dim3 grid, dim3 block, size_t lds_bytes, const std::function<void()>
                         if (!g_alive[i]) continue;
                         g_current = i;
                         g_thread = g_lane_idx[i];
-                        swapcontext(&g_scheduler, &g_lane_ctx[i]);
+                        hostsim_switch(&g_scheduler_sp, g_lane_sp[i]);
                         left += g_alive[i];
                     }
                     if (left > 0 && g_progress == before) {
