@@ -19,7 +19,7 @@ OUT = os.path.join(HERE, "_build")
 LIB = os.path.join(OUT, "libflexhip_hostsim.so")
 CLANG = "/opt/rocm/lib/llvm/bin/clang++"
 SOURCES = ("rmsnorm.hip", "rope.hip", "glu.hip", "softmax_ce.hip", "adamw.hip", "moe_route.hip", "moe_data.hip", "embed.hip",
-           "gemm.hip", "gemm_glu.hip", "gemm_ksum.hip", "gemm_segments.hip", "grouped_gemm.hip")
+           "gemm.hip", "gemm_glu.hip", "gemm_ksum.hip", "gemm_segments.hip", "grouped_gemm.hip", "stream.hip")
 HEADERS = ("common.h", "gemm_core.h", "gemm_core2.h")
 
 
