@@ -73,3 +73,17 @@ def test_zero_sized_problems_are_no_ops(ctx):
     L = sim.lib()
     for M, N, K in ((0, 8, 8), (8, 0, 8), (8, 8, 0)):
         assert L.dispatch_matmul(ctx, 0, M, N, K, 0, 8, 0, 8, 0, 8, 0, 8, 0, 0, 2, 2, 2, 2, 0, 1.0, 0.0, 0, 0) == 0
+
+
+def test_random_shapes_layouts_and_paddings(ctx):
+    """A sweep nobody chose by hand: any M, N, K (odd ones take the generic kernel), any layout, rows wider
+    than needed, accumulation or not, with or without a workspace.  Every operand ends at a guard page."""
+    g = torch.Generator().manual_seed(2024)
+    r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    for case in range(48):
+        multiple = 8 if case % 3 else 1
+        M, N, K = (r(1, 40) * multiple for _ in range(3))
+        if case % 8 == 0:
+            K = r(1, 20) * 64 + r(0, 7) * 8                  # long enough for several K-steps and a tail
+        _matmul(ctx, M, N, K, r(0, 1), r(0, 1), ddt=(BF, F32)[r(0, 1)], beta=float(r(0, 1)), alpha=(1.0, 0.5)[r(0, 1)],
+                pad=r(0, 2) * 8, ws_floats=(1 << 18) * r(0, 1), seed=case)

@@ -229,3 +229,44 @@ def test_fused_dense_forms():
     assert L.fx_gemm_ksum(2, arr([P(a) for a in gA]), i64(Ks), 0, arr([P(w) for w in gW]), i64(Ks), 1, (ctypes.c_int * 2)(*Ks), None, 72,
                           P(out), 72, M, 72, 1.0, 0.0, 2, 2, None) == 0
     _close(out, sum(a.float() @ w.float().t() for a, w in zip(As, Ws)).to(BF))
+
+
+def test_random_routings_and_shapes():
+    """Expert counts drawn at random (many zeros, single rows, a few hundred), N and K any multiple of 8:
+    rows GEMM and weight gradient on guard-paged buffers against per-expert fp32 products."""
+    g = torch.Generator().manual_seed(77)
+    r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    L = sim.lib()
+    for case in range(16):
+        E = r(1, 9)
+        counts = torch.tensor([(0, 1, r(2, 40), r(100, 700))[r(0, 3)] for _ in range(E)], dtype=torch.int32)
+        if case % 4 == 0:
+            counts[r(0, E - 1)] = r(400, 900)                   # one large expert: the 256-row tile form may be picked
+        rows = int(counts.sum())
+        if rows == 0:
+            counts[0] = 5
+            rows = 5
+        N, K = r(1, 40) * 8, r(1, 30) * 8
+        A = torch.randn(rows, K, generator=g).to(BF)
+        B = torch.randn(E, N, K, generator=g).to(BF)
+        ws, ws_bytes = _ws(E, rows)
+        D = G(torch.full((rows, N), 2.0, dtype=BF))
+        assert L.fx_grouped_gemm_rows(P(G(A)), K, P(G(B)), K, N * K, 1, None, N, P(D), N, P(G(counts)), E, rows, N, K, 1.0, 0.0, 2, P(ws),
+                                      ws_bytes, None) == 0
+        ref, off = torch.empty(rows, N), 0
+        for e in range(E):
+            c = int(counts[e])
+            ref[off:off + c] = A[off:off + c].float() @ B[e].float().t()
+            off += c
+        _close(D, ref.to(BF))
+        Bw = torch.randn(rows, N, generator=g).to(BF)
+        g0 = torch.randn(E, K, N, generator=g)
+        Gd = G(g0)
+        assert L.fx_grouped_gemm_wgrad(P(G(A)), K, P(G(Bw)), N, P(Gd), N, K * N, 0, P(G(counts)), E, rows, K, N, 1.0, 1.0, 2, P(ws), ws_bytes,
+                                       None, 0, None, 0, None) == 0
+        refg, off = g0.clone(), 0
+        for e in range(E):
+            c = int(counts[e])
+            refg[e] += A[off:off + c].float().t() @ Bw[off:off + c].float()
+            off += c
+        torch.testing.assert_close(Gd, refg, rtol=1e-4, atol=1e-3)
