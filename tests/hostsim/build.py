@@ -23,6 +23,15 @@ SOURCES = ("rmsnorm.hip", "rope.hip", "glu.hip", "softmax_ce.hip", "adamw.hip", 
 HEADERS = ("common.h", "gemm_core.h", "gemm_core2.h")
 
 
+def _marker():
+    import pytest
+
+    return pytest.mark.skipif(not os.path.exists(CLANG), reason=f"the host simulation is compiled with {CLANG}")
+
+
+needs_host_clang = _marker()
+
+
 def _match_forward(text, i, open_ch, close_ch):
     """Index just past the bracket that closes the one at ``text[i]``."""
     depth = 0

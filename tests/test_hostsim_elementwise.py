@@ -12,6 +12,10 @@ from oracle import glu as o_glu
 from oracle import rope as o_rope
 from tests.hostsim import sim
 
+from tests.hostsim.build import needs_host_clang
+
+pytestmark = needs_host_clang
+
 BF, F16, F32 = torch.bfloat16, torch.float16, torch.float32
 
 

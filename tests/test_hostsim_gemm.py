@@ -11,6 +11,10 @@ import torch
 
 from tests.hostsim import sim
 
+from tests.hostsim.build import needs_host_clang
+
+pytestmark = needs_host_clang
+
 BF, F16, F32 = torch.bfloat16, torch.float16, torch.float32
 G, P = sim.guard, sim.p
 

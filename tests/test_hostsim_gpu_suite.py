@@ -10,6 +10,10 @@ import re
 import subprocess
 import sys
 
+from tests.hostsim.build import needs_host_clang
+
+pytestmark = needs_host_clang
+
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 

@@ -13,6 +13,10 @@ import torch
 from oracle import moe as o_moe
 from tests.hostsim import sim
 
+from tests.hostsim.build import needs_host_clang
+
+pytestmark = needs_host_clang
+
 BF, F32 = torch.bfloat16, torch.float32
 G, P = sim.guard, sim.p
 

@@ -11,6 +11,10 @@ from oracle import linear_ce as o_ce
 from oracle import moe as o_moe
 from tests.hostsim import sim
 
+from tests.hostsim.build import needs_host_clang
+
+pytestmark = needs_host_clang
+
 BF, F32 = torch.bfloat16, torch.float32
 G = sim.guard
 P = sim.p

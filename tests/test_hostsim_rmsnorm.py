@@ -9,6 +9,10 @@ import torch
 from oracle import rmsnorm as o_norm
 from tests.hostsim import sim
 
+from tests.hostsim.build import needs_host_clang
+
+pytestmark = needs_host_clang
+
 BF = torch.bfloat16
 
 

@@ -9,6 +9,10 @@ import textwrap
 
 import os
 
+from tests.hostsim.build import needs_host_clang
+
+pytestmark = needs_host_clang
+
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
