@@ -73,7 +73,7 @@ def _parse():
     ap.add_argument("--no-extra", action="store_true", help="skip the non-headline configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--only", default="", help="comma-separated subset of the non-headline configurations "
-                                               "(c1, c3, c4, c5, moe_ref, ffn, attn, act, disp, probe) to run, e.g. for a profiler pass")
+                                               "(c1, c3, c4, c5, moe_ref, ffn, attn, act, disp, probe, a15) to run, e.g. for a profiler pass")
     return ap.parse_args()
 
 
@@ -941,6 +941,61 @@ def run_cpu_baselines(torch, only):
         rows.append(row("c5.cpu_baseline moe block fwd+bwd", 18 * T * K * d * F + 6 * T * d * E, "TFLOP/s", sec, runs,
                         "CPU oracle on 1/16 of the block: 512 tokens, 8 experts, top-8 (512 rows per expert as in the "
                         "full block)"))
+    if want("a15"):
+        rows += run_dp_solver(model)
+    return rows
+
+
+def run_dp_solver(cpu_model):
+    """The save-level solver (host code) beside the reference's own C solver, compiled from the
+    reference's source under oracle/_ref: one planning problem of 32 layers x 8 chunks, 4 options per
+    task, 8 activation slots, 0.1 ms ticks.  Both must return the same option vector."""
+    import ctypes
+
+    import numpy as np
+
+    from flextrain_amd._lib import lib
+
+    T, k, N, scale = 256, 4, 8, 10
+    rng = np.random.default_rng(15)
+    compute = rng.uniform(3.0, 9.0, T)
+    durations = np.ascontiguousarray(np.sort(rng.uniform(0.5, 12.0, (T, k)), axis=1))
+    sizes = np.ascontiguousarray(np.sort(rng.uniform(1.0, 100.0, (T, k)), axis=1))
+    deadline = float(compute.sum() + durations.max(axis=1).sum() + 1000.0)
+
+    def bind(so):
+        so.solve_scheduler.restype = ctypes.c_double
+        so.solve_scheduler.argtypes = [ctypes.c_int] * 3 + [ctypes.c_void_p] * 3 + [ctypes.c_double, ctypes.c_int,
+                                                                                     ctypes.c_int, ctypes.c_void_p]
+        so.compute_buf_size.restype = ctypes.c_int
+        so.compute_buf_size.argtypes = [ctypes.c_int] * 3 + [ctypes.c_void_p] * 2 + [ctypes.c_double, ctypes.c_int]
+        return so
+
+    def solve_with(so):
+        buf = so.compute_buf_size(T, N, k, compute.ctypes.data, durations.ctypes.data, deadline, scale)
+        choices = np.zeros(T, dtype=np.int32)
+        value = [0.0]
+
+        def once():
+            value[0] = so.solve_scheduler(T, N, k, compute.ctypes.data, durations.ctypes.data, sizes.ctypes.data,
+                                          deadline, scale, buf, choices.ctypes.data)
+
+        sec, runs = _cpu_time(once, 0.5, max_runs=2000)
+        return sec, runs, value[0], choices
+
+    shape = f"T {T} tasks x {k} options, {N} slots, {scale} ticks/ms"
+    sec, runs, value, choices = solve_with(lib())
+    rows = [{"op": f"a15.save-level solver, host C++ ({shape})", "algorithmic": None, "ms": round(sec * 1e3, 5),
+             "achieved": round(1.0 / sec, 1), "unit": "solves/s", "frac": None, "cores": 1, "cpu_model": cpu_model,
+             "sample": f"median of {runs} solves"}]
+    ref_path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "oracle", "_ref", "libts_ref.so")
+    if os.path.exists(ref_path):
+        rsec, rruns, rvalue, rchoices = solve_with(bind(ctypes.CDLL(ref_path)))
+        rows.append({"op": f"a15.cpu_baseline save-level solver, the reference's C source compiled ({shape})",
+                     "algorithmic": None, "ms": round(rsec * 1e3, 5), "achieved": round(1.0 / rsec, 1), "unit": "solves/s",
+                     "frac": None, "cores": 1, "cpu_model": cpu_model, "kind": "reference",
+                     "same_answer": bool(value == rvalue and np.array_equal(choices, rchoices)),
+                     "sample": f"median of {rruns} solves; the product solver takes {sec / rsec:.2f} of its time"})
     return rows
 
 
@@ -1154,6 +1209,10 @@ def main():
         brief("ffn.down gemm [", "ffn.down"), brief("ffn.down gemm, vendor", "ffn.down vendor"),
         brief("ffn.dense block fwd+bwd", "ffn.block"), brief("attn.projections fwd+bwd", "attn.proj"),
         brief("probe.save-level", "gemm8192^3")) if t is not None]
+    solver = [r for r in op_rows if r["op"].startswith("a15.")]
+    if solver:
+        summary.append("a15.solver " + " vs ".join(f"{r['ms']}ms" + (" (reference, same answer)" if r.get("same_answer") else "")
+                                                  for r in solver))
     summary += [f"{r['op']}: {r['error']}" for r in op_rows if "error" in r]
 
     result = {

@@ -33,13 +33,6 @@
 
 namespace {
 
-constexpr double kUnreached = -1.0e18;
-
-struct Step {           // how the best state with a given finish time was reached
-    int8_t option;
-    int32_t from;       // absolute finish time of the predecessor state
-};
-
 struct Ticks {
     std::vector<int> arrival, limit, dur;  // dur is T*k
 };
@@ -69,6 +62,36 @@ Ticks to_ticks(int T, int N, int k, const double* compute, const double* duratio
     return tk;
 }
 
+// The two inner loops are built once per vector width and picked by the CPU the library runs on; every
+// build gives the same results (no reassociation, compares and selects only).  Defining the macro empty
+// builds the single baseline form, e.g. to compare the forms with each other.
+#ifndef FX_VECTOR_BUILDS
+#define FX_VECTOR_BUILDS __attribute__((target_clones("avx512f", "avx2", "default")))
+#endif
+
+// One option of one task over the part of the band that was still transmitting at the arrival: a state
+// with finish time t becomes finish time t + dur with the option's value added.  cur and nxt are already
+// shifted so that element j of both is the same new finish time.  Strictly greater only: an earlier
+// writer (a lower option) keeps a tie.  The pick is kept as wide as the values so that the loop is one
+// compare and two blends per vector.
+FX_VECTOR_BUILDS
+void relax(const double* __restrict__ cur, double* __restrict__ nxt, int64_t* __restrict__ pick, int n, double value,
+           int64_t option) {
+    for (int j = 0; j < n; ++j) {
+        const double cand = cur[j] + value;
+        const bool better = cand > nxt[j];
+        nxt[j] = better ? cand : nxt[j];
+        pick[j] = better ? option : pick[j];
+    }
+}
+
+FX_VECTOR_BUILDS
+void narrow(const int64_t* __restrict__ pick, uint8_t* __restrict__ out, int n) {
+    for (int j = 0; j < n; ++j) out[j] = (uint8_t)pick[j];
+}
+
+constexpr int64_t kFromIdle = 0x80;   // the state was reached from the link-idle predecessor of its task
+
 }  // namespace
 
 extern "C" double solve_scheduler(int T, int N, int k, const double* compute, const double* durations,
@@ -76,17 +99,26 @@ extern "C" double solve_scheduler(int T, int N, int k, const double* compute, co
                                   int* out_choices) {
     if (T <= 0 || k <= 0 || k > 127 || buf_size <= 0 || !compute || !durations || !sizes || !out_choices) return 0.0;
     const Ticks tk = to_ticks(T, N, k, compute, durations, deadline, time_scale);
+    constexpr double kNone = -std::numeric_limits<double>::infinity();   // stays "unreached" under any addition
 
-    // band of the current states: value[t - lo] for finish times lo..hi
-    std::vector<double> cur(1, 0.0), nxt;
+    // Band of the current states: cur[t - lo] for finish times lo..hi.  Every kept finish time lies
+    // within buf_size ticks of the window origin, so two buffers of buf_size values alternate.
+    std::vector<double> store_a((size_t)buf_size, kNone), store_b((size_t)buf_size, kNone);
+    std::vector<int64_t> pick((size_t)buf_size);
+    double* const store[2] = {store_a.data(), store_b.data()};
+    int cur_in = 0;                  // which buffer holds the current band
+    double* cur = store[0];
+    cur[0] = 0.0;
     int lo = 0, hi = 0;
     int origin = 0;  // absolute tick of the reference window's index 0
-    std::vector<std::vector<Step>> trace(T);
-    std::vector<int> trace_lo(T);
+    // How each state was reached, one byte per state and task: the option, and whether the predecessor
+    // was the idle one (kept per task) or the busy one (its finish time is this one minus the duration).
+    std::vector<uint8_t> trace;
+    std::vector<size_t> trace_at(T);
+    std::vector<int> trace_lo(T), idle_from(T);
 
     for (int i = 0; i < T; ++i) {
         const int a = tk.arrival[i];
-        const int lim = tk.limit[i];
         const int* dur = &tk.dur[(size_t)i * k];
         const double* val = &sizes[(size_t)i * k];
         if (a - origin >= buf_size / 2 && lo > origin) origin = lo;
@@ -94,59 +126,65 @@ extern "C" double solve_scheduler(int T, int N, int k, const double* compute, co
         int longest = 0;
         for (int o = 0; o < k; ++o) longest = dur[o] > longest ? dur[o] : longest;
 
-        // best predecessor that leaves the link idle at the arrival (finish <= a)
-        double idle_best = kUnreached;
-        int idle_from = 0;
+        // best predecessor that leaves the link idle at the arrival (finish <= a), earliest first
+        double idle_best = kNone;
         for (int t = lo; t <= hi && t <= a; ++t) {
-            if (cur[t - lo] > idle_best) { idle_best = cur[t - lo]; idle_from = t; }
+            if (cur[t - lo] > idle_best) { idle_best = cur[t - lo]; idle_from[i] = t; }
         }
 
         const int busy_first = a + 1 > lo ? a + 1 : lo;           // predecessors still transmitting at a
-        const int out_lo = (a < lo ? a : lo) + 1;                 // earliest conceivable finish
-        const int out_hi = (a > hi ? a : hi) + longest;
-        nxt.assign((size_t)(out_hi - out_lo + 1), kUnreached);
-        std::vector<Step>& steps = trace[i];
-        steps.assign(nxt.size(), Step{0, 0});
-        trace_lo[i] = out_lo;
-        int new_lo = std::numeric_limits<int>::max(), new_hi = -1;
-
-        auto offer = [&](int finish, double total, int option, int from) {
-            const int rel = finish - origin;
-            if (finish > lim || rel < 0 || rel >= buf_size) return;
-            double& slot = nxt[finish - out_lo];
-            if (total > slot) {
-                slot = total;
-                steps[finish - out_lo] = Step{(int8_t)option, from};
-                if (finish < new_lo) new_lo = finish;
-                if (finish > new_hi) new_hi = finish;
-            }
-        };
+        // finish times this task can reach and may keep: before its deadline, inside the window
+        int out_lo = (a < lo ? a : lo) + 1;
+        int out_hi = (a > hi ? a : hi) + longest;
+        if (out_lo < origin) out_lo = origin;
+        if (out_hi > tk.limit[i]) out_hi = tk.limit[i];
+        if (out_hi > origin + buf_size - 1) out_hi = origin + buf_size - 1;
+        if (out_hi < out_lo) return 0.0;
+        const int width = out_hi - out_lo + 1;
+        double* nxt = store[cur_in ^ 1];
+        for (int j = 0; j < width; ++j) nxt[j] = kNone;
+        for (int j = 0; j < width; ++j) pick[j] = 0;
 
         for (int o = 0; o < k; ++o) {
-            if (idle_best > kUnreached) offer(a + dur[o], idle_best + val[o], o, idle_from);
-            for (int t = busy_first; t <= hi; ++t) {
-                const double v = cur[t - lo];
-                if (v > kUnreached) offer(t + dur[o], v + val[o], o, t);
+            const int d = dur[o];
+            const int f_idle = a + d;
+            if (idle_best > kNone && f_idle >= out_lo && f_idle <= out_hi && idle_best + val[o] > nxt[f_idle - out_lo]) {
+                nxt[f_idle - out_lo] = idle_best + val[o];
+                pick[f_idle - out_lo] = o | kFromIdle;
             }
+            const int f0 = busy_first + d > out_lo ? busy_first + d : out_lo;
+            const int f1 = hi + d < out_hi ? hi + d : out_hi;
+            if (f1 >= f0) relax(cur + (f0 - d - lo), nxt + (f0 - out_lo), pick.data() + (f0 - out_lo), f1 - f0 + 1, val[o], o);
         }
-        if (new_hi < 0) return 0.0;  // no option of this task meets its deadline
 
-        // keep the reached part of the band
-        cur.assign(nxt.begin() + (new_lo - out_lo), nxt.begin() + (new_hi - out_lo + 1));
-        lo = new_lo;
-        hi = new_hi;
+        int first = 0, last = width - 1;
+        while (first < width && !(nxt[first] > kNone)) ++first;
+        if (first == width) return 0.0;  // no option of this task meets its deadline
+        while (!(nxt[last] > kNone)) --last;
+
+        trace_at[i] = trace.size();
+        trace_lo[i] = out_lo + first;
+        trace.resize(trace.size() + (size_t)(last - first + 1));
+        narrow(pick.data() + first, trace.data() + trace_at[i], last - first + 1);
+
+        // the reached part of the band becomes the current one; the other buffer is written next
+        cur_in ^= 1;
+        cur = nxt + first;
+        lo = out_lo + first;
+        hi = out_lo + last;
     }
 
-    double best = kUnreached;
+    double best = kNone;
     int at = -1;
     for (int t = lo; t <= hi; ++t) {
         if (cur[t - lo] > best) { best = cur[t - lo]; at = t; }
     }
     if (at < 0) return 0.0;
     for (int i = T - 1; i >= 0; --i) {
-        const Step s = trace[i][at - trace_lo[i]];
-        out_choices[i] = s.option;
-        at = s.from;
+        const uint8_t how = trace[trace_at[i] + (size_t)(at - trace_lo[i])];
+        const int option = how & 0x7f;
+        out_choices[i] = option;
+        at = (how & kFromIdle) ? idle_from[i] : at - tk.dur[(size_t)i * k + option];
     }
     return best;
 }

@@ -151,3 +151,48 @@ def test_random_problems_against_compiled_reference():
             assert choices == rchoices.tolist(), trial
             checked += 1
     assert checked > 50
+
+
+@pytest.mark.parametrize("flags", [["-DFX_VECTOR_BUILDS="], ["-DFX_VECTOR_BUILDS=", "-mavx2"]], ids=["baseline", "avx2"])
+def test_every_vector_build_of_the_inner_loops_gives_the_same_answer(flags, tmp_path):
+    """The library picks a build of the two inner loops by the CPU it runs on; the other builds, compiled
+    here as the only one, must return the same values and option vectors (ties included: integer sizes)."""
+    import shutil
+    import subprocess
+
+    cxx = shutil.which("g++")
+    if cxx is None:
+        pytest.skip("no g++")
+    if "-mavx2" in flags and "avx2" not in open("/proc/cpuinfo").read():
+        pytest.skip("no AVX2 on this host")
+    root = os.path.join(HERE, "..")
+    so = str(tmp_path / "libsched_variant.so")
+    subprocess.run([cxx, "-O3", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include",
+                    "-I" + os.path.join(root, "include"), *flags,
+                    os.path.join(root, "flextrain_amd", "csrc", "scheduler.cpp"), "-o", so], check=True)
+    alt = ctypes.CDLL(so)
+    alt.solve_scheduler.argtypes = [ctypes.c_int] * 3 + [ctypes.c_void_p] * 3 + [ctypes.c_double, ctypes.c_int, ctypes.c_int,
+                                                                                 ctypes.c_void_p]
+    alt.solve_scheduler.restype = ctypes.c_double
+    rng = np.random.default_rng(41)
+    feasible = 0
+    for trial in range(150):
+        T, k, N = int(rng.integers(1, 300)), int(rng.integers(1, 6)), int(rng.integers(2, 14))
+        compute = rng.uniform(4.0, 12.0, size=T)
+        durations = rng.uniform(0.5, 18.0, size=(T, k))
+        sizes = rng.integers(1, 5, size=(T, k)).astype(np.float64) if trial % 2 else np.round(durations * 3.0, 2)
+        deadline = float(compute.sum() + durations.max(axis=1).sum() + 1000.0)
+        scale = 10 if trial % 5 else 100
+        c = dict(compute=compute, durations=durations, sizes=sizes, deadline=deadline, time_scale=scale, N=N, buf_size=None)
+        c["buf_size"] = lib().compute_buf_size(T, N, k, compute.ctypes.data, durations.ctypes.data, deadline, scale)
+        if trial % 7 == 0:
+            c["buf_size"] = 256                 # a window narrower than the band: states are dropped
+        _, val, choices = _product(c)
+        achoices = np.full(T, -1, dtype=np.int32)
+        aval = alt.solve_scheduler(T, N, k, compute.ctypes.data, durations.ctypes.data, sizes.ctypes.data, deadline, scale,
+                                   c["buf_size"], achoices.ctypes.data)
+        assert val == aval, trial
+        if val != 0.0:
+            feasible += 1
+            assert choices == achoices.tolist(), trial
+    assert feasible > 50
