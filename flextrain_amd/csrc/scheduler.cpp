@@ -94,21 +94,20 @@ constexpr int64_t kFromIdle = 0x80;   // the state was reached from the link-idl
 
 }  // namespace
 
-extern "C" double solve_scheduler(int T, int N, int k, const double* compute, const double* durations,
-                                  const double* sizes, double deadline, int time_scale, int buf_size,
-                                  int* out_choices) {
+static double solve(int T, int N, int k, const double* compute, const double* durations, const double* sizes,
+                    double deadline, int time_scale, int buf_size, int* out_choices) {
     if (T <= 0 || k <= 0 || k > 127 || buf_size <= 0 || !compute || !durations || !sizes || !out_choices) return 0.0;
     const Ticks tk = to_ticks(T, N, k, compute, durations, deadline, time_scale);
     constexpr double kNone = -std::numeric_limits<double>::infinity();   // stays "unreached" under any addition
 
-    // Band of the current states: cur[t - lo] for finish times lo..hi.  Every kept finish time lies
-    // within buf_size ticks of the window origin, so two buffers of buf_size values alternate.
-    std::vector<double> store_a((size_t)buf_size, kNone), store_b((size_t)buf_size, kNone);
-    std::vector<int64_t> pick((size_t)buf_size);
-    double* const store[2] = {store_a.data(), store_b.data()};
+    // Band of the current states: cur[t - lo] for finish times lo..hi.  Two buffers alternate; the one
+    // that is written next holds nothing live and grows to the width the task can reach (at most
+    // buf_size: every kept finish time lies within buf_size ticks of the window origin).
+    std::vector<double> store[2];
+    std::vector<int64_t> pick;
     int cur_in = 0;                  // which buffer holds the current band
-    double* cur = store[0];
-    cur[0] = 0.0;
+    store[0].assign(1, 0.0);
+    const double* cur = store[0].data();
     int lo = 0, hi = 0;
     int origin = 0;  // absolute tick of the reference window's index 0
     // How each state was reached, one byte per state and task: the option, and whether the predecessor
@@ -138,12 +137,12 @@ extern "C" double solve_scheduler(int T, int N, int k, const double* compute, co
         int out_hi = (a > hi ? a : hi) + longest;
         if (out_lo < origin) out_lo = origin;
         if (out_hi > tk.limit[i]) out_hi = tk.limit[i];
-        if (out_hi > origin + buf_size - 1) out_hi = origin + buf_size - 1;
+        if ((int64_t)out_hi > (int64_t)origin + buf_size - 1) out_hi = (int)((int64_t)origin + buf_size - 1);
         if (out_hi < out_lo) return 0.0;
         const int width = out_hi - out_lo + 1;
-        double* nxt = store[cur_in ^ 1];
-        for (int j = 0; j < width; ++j) nxt[j] = kNone;
-        for (int j = 0; j < width; ++j) pick[j] = 0;
+        store[cur_in ^ 1].assign((size_t)width, kNone);
+        pick.assign((size_t)width, 0);
+        double* nxt = store[cur_in ^ 1].data();
 
         for (int o = 0; o < k; ++o) {
             const int d = dur[o];
@@ -187,6 +186,16 @@ extern "C" double solve_scheduler(int T, int N, int k, const double* compute, co
         at = (how & kFromIdle) ? idle_from[i] : at - tk.dur[(size_t)i * k + option];
     }
     return best;
+}
+
+extern "C" double solve_scheduler(int T, int N, int k, const double* compute, const double* durations,
+                                  const double* sizes, double deadline, int time_scale, int buf_size,
+                                  int* out_choices) {
+    try {
+        return solve(T, N, k, compute, durations, sizes, deadline, time_scale, buf_size, out_choices);
+    } catch (...) {      // out of memory: "no schedule", as every other failure; nothing is thrown across the C ABI
+        return 0.0;
+    }
 }
 
 // Window width for solve_scheduler: a power of two, at least 2048, that covers the widest

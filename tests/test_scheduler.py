@@ -196,3 +196,12 @@ def test_every_vector_build_of_the_inner_loops_gives_the_same_answer(flags, tmp_
             feasible += 1
             assert choices == achoices.tolist(), trial
     assert feasible > 50
+
+
+def test_a_huge_window_costs_nothing():
+    """The window width only bounds which states are kept: memory follows the band that the tasks can
+    reach, so the largest window a caller can name gives the unwindowed answer at once."""
+    c = dict(next(c for c in CASES if c["name"] == "tradeoff_64x4"))
+    _, val, choices = _product(c, buf_size=(1 << 31) - 1)
+    oval, ochoices = o_dp.solve_scheduler(c["compute"], c["durations"], c["sizes"], c["deadline"], c["time_scale"], c["N"])
+    assert val == oval == 35700.0 and choices == ochoices.tolist()
