@@ -1243,4 +1243,12 @@ def main():
 
 
 if __name__ == "__main__":
-    main()
+    try:
+        main()
+    except Exception as exc:  # noqa: BLE001 - the headline itself failed: say so in the one line, then fail
+        import traceback
+
+        traceback.print_exc()
+        print(json.dumps({"metric": METRIC, "value": None, "unit": "GB/s", "n_gpus": 1,
+                          "error": f"{type(exc).__name__}: {exc}"}))
+        sys.exit(1)
