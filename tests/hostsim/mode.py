@@ -59,13 +59,28 @@ class _Stream:
         return True
 
 
+def _behind_a_guard_page(t):
+    """A fresh, dense tensor moves to storage that ends at an inaccessible page (released with the tensor):
+    a kernel that reads or writes past the end of an operand, an output or a workspace then ends the test
+    with a segmentation fault instead of passing unnoticed.  Anything else is returned as it is."""
+    from . import sim
+
+    if (not isinstance(t, torch.Tensor) or type(t) is not torch.Tensor or t.requires_grad or t.grad_fn is not None
+            or t.layout != torch.strided or t.device.type != "cpu" or t.numel() == 0 or not t.is_contiguous()
+            or t.dtype in (torch.bool, torch.complex64, torch.complex128)):
+        return t
+    return sim.guard(t, align=16, keep=False)       # 16-byte aligned starts, as every device allocation has
+
+
 def _host_only(fn):
     def wrapped(*args, **kwargs):
         kwargs.pop("pin_memory", None)
         dev = kwargs.get("device")
         if dev is not None and torch.device(dev).type == "cuda":
             kwargs["device"] = "cpu"
-        return fn(*args, **kwargs)
+        if kwargs.get("out") is not None:
+            return fn(*args, **kwargs)
+        return _behind_a_guard_page(fn(*args, **kwargs))
     return wrapped
 
 
@@ -103,10 +118,19 @@ def activate():
     # the host original that the oracle is given afterwards); on one device Tensor.to returns the tensor itself
     plain_to = torch.Tensor.to
 
+    plain_clone = torch.Tensor.clone
+
     def to(self, *args, **kwargs):
         out = plain_to(self, *args, **kwargs)
         moved = "device" in kwargs or any(isinstance(a, (torch.device, str)) for a in args)
-        return out.clone() if (out is self and moved) else out
+        if not moved:
+            return out
+        return _behind_a_guard_page(plain_clone(out) if out is self else out)
+
+    def clone(self, *args, **kwargs):
+        return _behind_a_guard_page(plain_clone(self, *args, **kwargs))
+
+    torch.Tensor.clone = clone
 
     torch.Tensor.to = to
     # every tensor is "on the GPU" except those the package's pinned-host allocator made
@@ -117,9 +141,10 @@ def activate():
         return any(base <= p < base + nbytes for base, (_, nbytes) in host_memory._PROCESS_PINNED.items())
 
     torch.Tensor.is_cuda = property(lambda self: not in_pinned_host_memory(self))
-    torch.Tensor.cpu = lambda self, *a, **k: self.clone()      # a device-to-host copy is a copy
+    torch.Tensor.cpu = lambda self, *a, **k: plain_clone(self)      # a device-to-host copy is a copy
     torch.Tensor.is_pinned = lambda self, device=None: True
     torch.Tensor.pin_memory = lambda self, device=None: self
     torch.Tensor.record_stream = lambda self, stream: None
-    for name in ("empty", "zeros", "ones", "full", "tensor", "randn", "rand", "arange"):
+    for name in ("empty", "zeros", "ones", "full", "tensor", "randn", "rand", "arange", "randint", "empty_like", "zeros_like",
+                 "ones_like", "full_like", "randn_like", "rand_like"):
         setattr(torch, name, _host_only(getattr(torch, name)))

@@ -13,7 +13,7 @@ from . import build as _build
 _PAGE = mmap.PAGESIZE
 _libc = ctypes.CDLL(None, use_errno=True)
 _libc.mprotect.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
-_keep = []          # the mappings live as long as the process: tensors made from them hold no reference
+_keep = []          # mappings of guard(..., keep=True): they live as long as the process
 _lib = None
 
 
@@ -33,20 +33,26 @@ def lib():
     return _lib
 
 
-def guard(t: torch.Tensor, align: int = 16) -> torch.Tensor:
+def guard(t: torch.Tensor, align: int = 16, keep: bool = True) -> torch.Tensor:
     """A copy of ``t`` (contiguous) whose last byte is followed, within ``align`` bytes, by a page that
-    may be neither read nor written; the page before the mapping's first is protected too."""
+    may be neither read nor written; the page before the mapping's first is protected too.  With ``keep``
+    the mapping lives as long as the process, so that a test may pass ``p(guard(x))`` of a temporary;
+    without it the tensor alone holds the mapping (``torch.frombuffer`` keeps its buffer) and releases it
+    when it dies."""
     t = t.detach().contiguous()
     nbytes = t.numel() * t.element_size()
-    body = (max(nbytes, 1) + _PAGE - 1) // _PAGE * _PAGE
+    if nbytes == 0:
+        return torch.empty_like(t)
+    body = (nbytes + _PAGE - 1) // _PAGE * _PAGE
     mm = mmap.mmap(-1, body + 2 * _PAGE)
-    base = ctypes.addressof(ctypes.c_char.from_buffer(mm))
+    probe = ctypes.c_char.from_buffer(mm)
+    base = ctypes.addressof(probe)
+    del probe
     if _libc.mprotect(base, _PAGE, 0) != 0 or _libc.mprotect(base + _PAGE + body, _PAGE, 0) != 0:
         raise OSError(ctypes.get_errno(), "mprotect")
     start = (_PAGE + body - nbytes) // align * align
-    _keep.append(mm)
-    if nbytes == 0:
-        return torch.empty_like(t)
+    if keep:
+        _keep.append(mm)
     out = torch.frombuffer(mm, dtype=t.dtype, count=t.numel(), offset=start).view(t.shape)
     out.copy_(t)
     return out

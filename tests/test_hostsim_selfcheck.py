@@ -40,3 +40,40 @@ def test_an_overrun_of_one_pack_dies_on_the_guard_page():
             print("survived")
         """)
         assert bad.returncode == -signal.SIGSEGV and "survived" not in bad.stdout, (victim, bad.returncode, bad.stderr[-500:])
+
+
+def test_tensors_of_the_simulated_gpu_suite_end_at_a_guard_page():
+    """With FLEXTRAIN_HOSTSIM=1 every tensor created, cloned or moved "to the device" is guarded: the same
+    overrun through the package's own ops dies there as well, and the tensor releases its pages when it dies."""
+    prologue = """
+        import os, sys
+        os.environ["FLEXTRAIN_HOSTSIM"] = "1"
+        sys.path.insert(0, "tests")
+        import torch
+        from hostsim import mode
+        mode.ACTIVE = True
+        mode.activate()
+        from flextrain_amd._lib import lib
+        n = 4096
+        dev = torch.device("cpu")               # what the tests' device fixture hands out in this mode
+    """
+    ok = _child(prologue + """
+        for _ in range(200):                    # 200 x 3 x 4 MB = 2.4 GB if the mappings were kept
+            a = torch.zeros(1 << 21, dtype=torch.bfloat16, device=dev)
+            b, c = a.clone(), torch.ones(1 << 21, dtype=torch.bfloat16).to(dev)
+        import resource
+        assert resource.getrusage(resource.RUSAGE_SELF).ru_maxrss < (1 << 20), "guarded tensors are not released"   # KiB
+        a, b, o = (torch.zeros(n, dtype=torch.bfloat16, device=dev) for _ in range(3))
+        assert lib().fx_glu_fwd(a.data_ptr(), b.data_ptr(), o.data_ptr(), n, 2, 2, 0, None) == 0
+        print("fine")
+    """)
+    assert ok.returncode == 0 and "fine" in ok.stdout, ok.stderr[-2000:]
+    for make in ('torch.zeros(n, dtype=torch.bfloat16, device=dev)', 'torch.zeros(n, dtype=torch.bfloat16).to(dev)',
+                 'torch.zeros(n, dtype=torch.bfloat16).clone()', 'torch.empty_like(torch.zeros(n, dtype=torch.bfloat16))'):
+        bad = _child(prologue + f"""
+        a, b = (torch.zeros(n + 8, dtype=torch.bfloat16, device=dev) for _ in range(2))
+        o = {make}
+        lib().fx_glu_fwd(a.data_ptr(), b.data_ptr(), o.data_ptr(), n + 8, 2, 2, 0, None)
+        print("survived")
+        """)
+        assert bad.returncode == -signal.SIGSEGV and "survived" not in bad.stdout, (make, bad.returncode, bad.stderr[-500:])
