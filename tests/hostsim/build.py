@@ -101,7 +101,8 @@ def rewrite_dynamic_lds(text):
 
 def rewrite_asm(text):
     """The three kinds of inline assembly in the GEMM code: the two LDS-DMA loads become calls of the
-    stand-in, the wait-count instructions (the stand-in load completes at once) become nothing."""
+    stand-in, which queues the copy; the wait-count instructions become the call that lets the lane's
+    queued copies land down to the count they name."""
     def one(m):
         body = m.group(1)
         if "global_load_lds_dwordx4 %1, off" in body:
@@ -109,7 +110,13 @@ def rewrite_asm(text):
         if "global_load_lds_dwordx4 %1, %2" in body:
             return "hostsim::lds_dma16(lds_addr, reinterpret_cast<const char*>(sbase) + lane_off);"
         assert "s_waitcnt" in body, f"inline assembly the host simulation has no stand-in for: {body[:80]}"
-        return "((void)0);"
+        count = re.search(r"vmcnt\((\d+|%0)\)", body)
+        if count is None:
+            return "((void)0);"
+        n = count.group(1)
+        if n == "%0":
+            n = re.search(r'"n"\((.*?)\)\s*:', body).group(1)
+        return f"hostsim::wait_vmcnt({n});"
     return re.sub(r"asm volatile\((.*?)\);", one, text)
 
 

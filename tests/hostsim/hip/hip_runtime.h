@@ -144,9 +144,32 @@ namespace hostsim {
 extern float (*g_wave_f32)[64][16];             // [wave][lane][8 of A, 8 of B]: operands published for a matrix instruction
 
 // global_load_lds_dwordx4: lane l of the wave copies 16 bytes from its global address to lds_addr + 16 l.
-// Completes at once (one of the orders the hardware may take; the kernels wait before they read).
+// The copy is made as LATE as the hardware may make it: it is queued, and lands only when the lane's own
+// `s_waitcnt vmcnt(n)` leaves at most n of its loads in flight (oldest first).  A kernel that reads a buffer
+// before its counted wait has covered the loads that fill it, or re-uses a buffer that loads are still in
+// flight to, computes from stale or overwritten data here and fails its comparison.  (Counting these loads
+// alone is the weaker guarantee: other vector memory operations in the window only make the real wait cover
+// more.)  Loads never waited for are dropped when the workgroup ends.
+struct PendingDma { unsigned lds; const void* src; };
+constexpr int kMaxPendingDma = 64;
+extern PendingDma g_dma[][kMaxPendingDma];
+extern int g_dma_first[], g_dma_count[];
+extern int g_dma_eager;     // 1: the other extreme, every copy lands at its issue (a load into a buffer that
+                            // lanes scheduled later still have to read then shows as wrong results)
 inline void lds_dma16(unsigned lds_addr, const void* gptr) {
-    memcpy(reinterpret_cast<void*>((uintptr_t)lds_addr + 16u * (flat_thread() & 63u)), gptr, 16);
+    const unsigned me = flat_thread();
+    if (g_dma_eager) { memcpy(reinterpret_cast<void*>((uintptr_t)lds_addr + 16u * (me & 63u)), gptr, 16); return; }
+    if (g_dma_count[me] == kMaxPendingDma) { fprintf(stderr, "hostsim: more than %d LDS loads in flight in one lane\n", kMaxPendingDma); abort(); }
+    g_dma[me][(g_dma_first[me] + g_dma_count[me]++) % kMaxPendingDma] = PendingDma{lds_addr + 16u * (me & 63u), gptr};
+}
+inline void wait_vmcnt(int n) {
+    const unsigned me = flat_thread();
+    while (g_dma_count[me] > n) {
+        const PendingDma& d = g_dma[me][g_dma_first[me]];
+        memcpy(reinterpret_cast<void*>((uintptr_t)d.lds), d.src, 16);
+        g_dma_first[me] = (g_dma_first[me] + 1) % kMaxPendingDma;
+        --g_dma_count[me];
+    }
 }
 
 // v_mfma_f32_32x32x16 (bf16 / f16): D = A (32 x 16) * B (16 x 32) + C.  Lane l supplies A[l % 32][8 (l / 32) .. + 7]

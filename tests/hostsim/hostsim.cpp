@@ -63,6 +63,9 @@ static unsigned g_alive_wave[MAX_LANES / 64], g_arrived_wave[MAX_LANES / 64], g_
 static unsigned long g_progress = 0;
 
 unsigned flat_thread() { return (unsigned)g_current; }
+PendingDma g_dma[MAX_LANES][kMaxPendingDma];
+int g_dma_first[MAX_LANES], g_dma_count[MAX_LANES];
+int g_dma_eager = 0;
 
 static void yield() { hostsim_switch(&g_lane_sp[g_current], g_scheduler_sp); }
 
@@ -124,6 +127,7 @@ void launch(dim3 grid, dim3 block, size_t lds_bytes, const std::function<void()>
                 for (int i = 0; i < lanes; ++i) {
                     g_lane_idx[i] = Idx{(unsigned)i % block.x, ((unsigned)i / block.x) % block.y, (unsigned)i / (block.x * block.y)};
                     g_alive[i] = 1;
+                    g_dma_first[i] = g_dma_count[i] = 0;
                     ++g_alive_wave[i >> 6];
                     // a fresh stack that hostsim_switch can "return" into: six saved registers, then lane_main as the
                     // return address, at the alignment a called function expects
@@ -155,3 +159,6 @@ void launch(dim3 grid, dim3 block, size_t lds_bytes, const std::function<void()>
 }
 
 }  // namespace hostsim
+
+// 0 (default): LDS loads land as late as their counted waits allow; 1: at their issue.
+extern "C" void hostsim_set_dma_eager(int eager) { hostsim::g_dma_eager = eager; }

@@ -21,6 +21,16 @@ BF, F32 = torch.bfloat16, torch.float32
 G, P = sim.guard, sim.p
 
 
+@pytest.fixture(autouse=True, params=["loads land late", "loads land early"])
+def dma_timing(request):
+    """Every test runs at both extremes of what the hardware may do with a load into LDS: landing only when
+    the issuing lane's counted wait says it must have (a read that the wait does not cover sees stale data),
+    and landing at its issue (a load into a buffer that other lanes still read shows as wrong results)."""
+    sim.lib().hostsim_set_dma_eager(int(request.param == "loads land early"))
+    yield
+    sim.lib().hostsim_set_dma_eager(0)
+
+
 def _counts(E, total, g, empty=()):
     w = torch.rand(E, generator=g) + 0.2
     for e in empty:
