@@ -29,8 +29,6 @@ template <> struct VecOf<float> { static constexpr int N = 4; typedef float type
 template <> struct VecOf<bf16>  { static constexpr int N = 8; typedef bf16  type __attribute__((ext_vector_type(8))); };
 template <> struct VecOf<f16>   { static constexpr int N = 8; typedef f16   type __attribute__((ext_vector_type(8))); };
 
-template <typename T> FX_DEV float to_f32(T v) { return (float)v; }
-template <typename T> FX_DEV T from_f32(float v) { return (T)v; }
 
 // Load/store `N` consecutive elements (N * sizeof(T) must be 16 or 32 bytes and
 // the address 16-byte aligned) converting to/from fp32 registers.
@@ -134,21 +132,6 @@ FX_DEV float group_max(float v) {
 #pragma unroll
     for (int off = W / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
     return v;
-}
-
-// Sum across `NWAVES` waves of a workgroup through LDS (smem needs NWAVES
-// floats).  All threads of the participating waves must call it.
-template <int NWAVES>
-FX_DEV float block_sum(float v, float* smem, int wave_in_group, int lane) {
-    v = group_sum<64>(v);
-    if (NWAVES == 1) return v;
-    __syncthreads();
-    if (lane == 0) smem[wave_in_group] = v;
-    __syncthreads();
-    float t = 0.f;
-#pragma unroll
-    for (int i = 0; i < NWAVES; ++i) t += smem[i];
-    return t;
 }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

@@ -66,6 +66,7 @@ unsigned flat_thread() { return (unsigned)g_current; }
 PendingDma g_dma[MAX_LANES][kMaxPendingDma];
 int g_dma_first[MAX_LANES], g_dma_count[MAX_LANES];
 int g_dma_eager = 0;
+static int g_reverse_schedule = 0;
 
 static void yield() { hostsim_switch(&g_lane_sp[g_current], g_scheduler_sp); }
 
@@ -141,7 +142,8 @@ void launch(dim3 grid, dim3 block, size_t lds_bytes, const std::function<void()>
                 while (left > 0) {
                     const unsigned long before = g_progress;
                     left = 0;
-                    for (int i = 0; i < lanes; ++i) {
+                    for (int slot = 0; slot < lanes; ++slot) {
+                        const int i = g_reverse_schedule ? lanes - 1 - slot : slot;
                         if (!g_alive[i]) continue;
                         g_current = i;
                         g_thread = g_lane_idx[i];
@@ -162,3 +164,8 @@ void launch(dim3 grid, dim3 block, size_t lds_bytes, const std::function<void()>
 
 // 0 (default): LDS loads land as late as their counted waits allow; 1: at their issue.
 extern "C" void hostsim_set_dma_eager(int eager) { hostsim::g_dma_eager = eager; }
+
+// Between two barriers the lanes of a workgroup run one after another: in ascending order (0, default) or
+// in descending order (1).  A value that one wave writes to LDS and another reads with no barrier in
+// between is read before it is written in one of the two orders.
+extern "C" void hostsim_set_reverse_schedule(int reverse) { hostsim::g_reverse_schedule = reverse; }

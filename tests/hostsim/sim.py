@@ -29,6 +29,7 @@ def lib():
             fn = getattr(handle, name, None)
             if fn is not None:
                 fn.restype, fn.argtypes = restype, argtypes
+        handle.hostsim_set_reverse_schedule(int(os.environ.get("HOSTSIM_LANE_ORDER", "ascending") == "descending"))
         _lib = handle
     return _lib
 
