@@ -16,14 +16,21 @@ unsigned char g_alive[MAX_LANES];
 constexpr size_t LDS_BYTES = 160 * 1024;
 static unsigned char* map_lds() {
     for (uintptr_t at = 0x40000000u; at < 0xF0000000u; at += 0x10000000u) {
-        void* p = mmap((void*)at, LDS_BYTES, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_FIXED_NOREPLACE, -1, 0);
-        if (p == (void*)at) return (unsigned char*)p;
-        if (p != MAP_FAILED) munmap(p, LDS_BYTES);
+        void* p = mmap((void*)at, LDS_BYTES + 4096, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_FIXED_NOREPLACE, -1, 0);
+        if (p == (void*)at) {
+            mprotect((unsigned char*)p + LDS_BYTES, 4096, PROT_NONE);     // the page after the LDS
+            return (unsigned char*)p;
+        }
+        if (p != MAP_FAILED) munmap(p, LDS_BYTES + 4096);
     }
     fprintf(stderr, "hostsim: no room below 4 GB for the LDS\n");
     abort();
 }
-unsigned char* g_dynamic_lds = map_lds();
+static unsigned char* const g_lds_region = map_lds();
+// The dynamic LDS of a launch ENDS where the region ends (16-byte aligned start, all the hardware promises),
+// so an access past the size the launch asked for hits the protected page; it starts every workgroup with
+// all bits set (NaN / -1), as unpredictable as what the previous workgroup left on the hardware.
+unsigned char* g_dynamic_lds = g_lds_region;
 static float g_wave_store[MAX_LANES / 64][64][16];
 float (*g_wave_f32)[64][16] = g_wave_store;
 
@@ -114,6 +121,7 @@ void launch(dim3 grid, dim3 block, size_t lds_bytes, const std::function<void()>
         g_stacks = (char*)mmap(nullptr, STACK_BYTES * MAX_LANES, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0);
         if (g_stacks == (char*)MAP_FAILED) { perror("hostsim: mmap"); abort(); }
     }
+    g_dynamic_lds = g_lds_region + LDS_BYTES - (lds_bytes + 15) / 16 * 16;
     g_body = &body;
     g_block_dim = block;
     g_grid_dim = grid;
@@ -122,6 +130,7 @@ void launch(dim3 grid, dim3 block, size_t lds_bytes, const std::function<void()>
         for (unsigned by = 0; by < grid.y; ++by)
             for (unsigned bx = 0; bx < grid.x; ++bx) {
                 g_block = Idx{bx, by, bz};
+                if (lds_bytes) memset(g_dynamic_lds, 0xFF, lds_bytes);
                 g_alive_block = (unsigned)lanes;
                 g_arrived_block = 0;
                 for (int w = 0; w < MAX_LANES / 64; ++w) { g_alive_wave[w] = 0; g_arrived_wave[w] = 0; }

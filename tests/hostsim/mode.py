@@ -72,7 +72,10 @@ def _behind_a_guard_page(t):
     return sim.guard(t, align=16, keep=False)       # 16-byte aligned starts, as every device allocation has
 
 
-def _host_only(fn):
+def _host_only(fn, poison=False):
+    """``poison``: memory that the caller did not initialise (torch.empty) reads as NaN / -1 (all bits set)
+    instead of the zeros a fresh mapping holds, so a kernel that consumes scratch memory or an output it
+    never wrote cannot pass by luck."""
     def wrapped(*args, **kwargs):
         kwargs.pop("pin_memory", None)
         dev = kwargs.get("device")
@@ -80,7 +83,10 @@ def _host_only(fn):
             kwargs["device"] = "cpu"
         if kwargs.get("out") is not None:
             return fn(*args, **kwargs)
-        return _behind_a_guard_page(fn(*args, **kwargs))
+        out = _behind_a_guard_page(fn(*args, **kwargs))
+        if poison and isinstance(out, torch.Tensor) and out.numel() and out.is_contiguous() and out.dtype != torch.bool:
+            out.view(-1).view(torch.uint8).fill_(0xFF)
+        return out
     return wrapped
 
 
@@ -147,4 +153,4 @@ def activate():
     torch.Tensor.record_stream = lambda self, stream: None
     for name in ("empty", "zeros", "ones", "full", "tensor", "randn", "rand", "arange", "randint", "empty_like", "zeros_like",
                  "ones_like", "full_like", "randn_like", "rand_like"):
-        setattr(torch, name, _host_only(getattr(torch, name)))
+        setattr(torch, name, _host_only(getattr(torch, name), poison=name in ("empty", "empty_like")))

@@ -51,7 +51,9 @@ def guard(t: torch.Tensor, align: int = 16, keep: bool = True) -> torch.Tensor:
     del probe
     if _libc.mprotect(base, _PAGE, 0) != 0 or _libc.mprotect(base + _PAGE + body, _PAGE, 0) != 0:
         raise OSError(ctypes.get_errno(), "mprotect")
-    start = (_PAGE + body - nbytes) // align * align
+    # HOSTSIM_GUARD_SIDE=front puts the tensor right after the protected first page instead: the check for
+    # accesses BEFORE a buffer (a negative index, an offset subtracted twice)
+    start = _PAGE if os.environ.get("HOSTSIM_GUARD_SIDE") == "front" else (_PAGE + body - nbytes) // align * align
     if keep:
         _keep.append(mm)
     out = torch.frombuffer(mm, dtype=t.dtype, count=t.numel(), offset=start).view(t.shape)
