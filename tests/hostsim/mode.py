@@ -12,23 +12,35 @@ import os
 
 import torch
 
+from .order import CLOCKS, OrderedLibrary
+
 ACTIVE = os.environ.get("FLEXTRAIN_HOSTSIM") == "1"
 
 
+def _current():
+    return torch.cuda.current_stream()
+
+
 class _Event:
+    """Completes at once (the simulated library finishes every launch and copy at the call); what it keeps is
+    the vector clock of its stream at ``record``, for the happens-before check of ``order.py``."""
+
     def __init__(self, *a, **k):
-        pass
+        self.clock = None
 
-    def record(self, *a, **k):
-        pass
+    def record(self, stream=None):
+        self.clock = CLOCKS.snapshot((stream or _current()).cuda_stream)
 
-    def wait(self, *a, **k):
-        pass
+    def wait(self, stream=None):
+        if self.clock is not None:
+            CLOCKS.wait((stream or _current()).cuda_stream, self.clock)
 
     def synchronize(self):
-        pass
+        if self.clock is not None:
+            CLOCKS.host_sync(self.clock)
 
     def query(self):
+        self.synchronize()          # "complete", and the host has now seen it
         return True
 
     def elapsed_time(self, other):
@@ -44,18 +56,21 @@ class _Stream:
         self.cuda_stream = 0x1000 * _Stream._handles       # a distinct non-null handle per stream object
 
     def synchronize(self):
-        pass
+        CLOCKS.host_sync(CLOCKS.snapshot(self.cuda_stream))
 
     def wait_stream(self, other):
-        pass
+        CLOCKS.wait(self.cuda_stream, CLOCKS.snapshot(other.cuda_stream))
 
     def wait_event(self, event):
-        pass
+        event.wait(self)
 
     def record_event(self, event=None):
-        return event or _Event()
+        event = event or _Event()
+        event.record(self)
+        return event
 
     def query(self):
+        self.synchronize()
         return True
 
 
@@ -95,7 +110,7 @@ def activate():
 
     from . import sim
 
-    _lib._lib = sim.lib()
+    _lib._lib = OrderedLibrary(sim.lib())
     default = _Stream()
     default.cuda_stream = 0
     current = [default]
@@ -114,7 +129,7 @@ def activate():
     torch.cuda.current_stream = lambda device=None: current[-1]
     torch.cuda.default_stream = lambda device=None: default
     torch.cuda.stream = stream_context
-    torch.cuda.synchronize = lambda device=None: None
+    torch.cuda.synchronize = lambda device=None: CLOCKS.host_sync()
     torch.cuda.Stream = _Stream
     torch.cuda.Event = _Event
     torch.cuda.memory_allocated = lambda device=None: 0

@@ -77,3 +77,47 @@ def test_tensors_of_the_simulated_gpu_suite_end_at_a_guard_page():
         print("survived")
         """)
         assert bad.returncode == -signal.SIGSEGV and "survived" not in bad.stdout, (make, bad.returncode, bad.stderr[-500:])
+
+
+def test_a_removed_wait_in_the_streamed_optimizer_step_is_reported():
+    """The happens-before check of the simulated run: the pipelined optimizer step over the layer rings passes
+    with many cross-stream pairs examined, and taking away any one class of its waits (the compute stream's
+    wait for a layer's fetches, the outbound stream's wait for the update, the inbound stream's wait before a
+    slot is refilled) raises StreamOrderError at the enqueue that is no longer ordered."""
+    prologue = """
+        import os, sys
+        os.environ["FLEXTRAIN_HOSTSIM"] = "1"
+        sys.path.insert(0, "tests")
+        import torch
+        from hostsim import mode, order
+        mode.ACTIVE = True
+        mode.activate()
+        import test_gpu_layer_ring as t
+        from flextrain_amd.layer_ring import ring_optimizer_step
+        from flextrain_amd.streams import EventBook, StreamBundle
+        dev = torch.device("cpu")
+        def run():
+            specs, buf = t._make(dev, 5, 2, 2, 7)
+            streams = StreamBundle.create(dev)
+            return streams, ring_optimizer_step(buf, streams, EventBook(), n_gpu_opt_layers=2, step_num=4, **t.HP)
+    """
+    ok = _child(prologue + """
+        assert run()[1] == 0
+        assert order.CLOCKS.checked > 50, order.CLOCKS.checked
+        print("fine", order.CLOCKS.checked)
+    """)
+    assert ok.returncode == 0 and "fine" in ok.stdout, ok.stderr[-2000:]
+    for role in ("compute", "outbound", "inbound"):
+        bad = _child(prologue + f"""
+        streams = StreamBundle.create(dev)
+        deaf = streams.{role}.cuda_stream
+        plain = order.CLOCKS.wait
+        order.CLOCKS.wait = lambda sid, clock: None if sid == deaf else plain(sid, clock)   # this stream waits for nothing
+        StreamBundle.create = classmethod(lambda cls, *a, **k: streams)
+        try:
+            run()
+            print("unnoticed")
+        except order.StreamOrderError as exc:
+            print("reported:", exc)
+        """)
+        assert bad.returncode == 0 and "reported:" in bad.stdout and "unnoticed" not in bad.stdout, (role, bad.stdout[-500:], bad.stderr[-1500:])
