@@ -120,6 +120,30 @@ def rewrite_asm(text):
     return re.sub(r"asm volatile\((.*?)\);", one, text)
 
 
+# Entry points whose launches take part in multi-stream schedules declare the bytes they read and write to
+# the happens-before check (order.cpp) before anything else: (pointer, bytes, is_write) triples.
+DECLARED_ACCESSES = {
+    "fx_adamw_step": [("g", "n * elem_size(g_dt)", 0), ("p", "n * elem_size(p_dt)", 1), ("m", "n * elem_size(state_dt)", 1),
+                      ("v", "n * elem_size(state_dt)", 1), ("p_bf16_out", "n * 2", 1)],
+}
+
+
+def rewrite_declared_accesses(text):
+    for name, accesses in DECLARED_ACCESSES.items():
+        m = re.search(r'extern "C" int ' + name + r"\(", text)
+        if m is None:
+            continue
+        brace = text.index("{", _match_forward(text, m.end() - 1, "(", ")"))
+        lo = ", ".join(f"(uint64_t)(uintptr_t)({ptr})" for ptr, _, _ in accesses)
+        nbytes = ", ".join(f"(uint64_t)(n > 0 ? ({size}) : 0)" for _, size, _ in accesses)
+        writes = ", ".join(str(w) for _, _, w in accesses)
+        snippet = (f"\n    {{ const uint64_t lo__[] = {{{lo}}}, bytes__[] = {{{nbytes}}}; const int write__[] = {{{writes}}};"
+                   f"\n      if (hostsim_order_enqueue((uint64_t)(uintptr_t)stream, \"{name}\", {len(accesses)}, lo__, bytes__, write__))"
+                   f" FX_FAIL(\"{name}: stream order violation (host simulation)\"); }}")
+        text = text[:brace + 1] + snippet + text[brace + 1:]
+    return text
+
+
 def rewrite_lockstep(text):
     """A GPU wave runs its lanes in lockstep, so a wave may stage values in LDS and read its neighbours'
     values back with no barrier in between; fibers do not.  The sources mark those points with comment lines
@@ -129,7 +153,7 @@ def rewrite_lockstep(text):
 
 def build(force=False):
     os.makedirs(OUT, exist_ok=True)
-    inputs = [os.path.join(CSRC, f) for f in SOURCES + HEADERS] + [os.path.join(HERE, "hostsim.cpp"),
+    inputs = [os.path.join(CSRC, f) for f in SOURCES + HEADERS] + [os.path.join(HERE, "hostsim.cpp"), os.path.join(HERE, "order.cpp"),
                                                                       os.path.join(HERE, "hip", "hip_runtime.h"), os.path.abspath(__file__)]
     if not force and os.path.exists(LIB) and all(os.path.getmtime(LIB) >= os.path.getmtime(p) for p in inputs):
         return LIB
@@ -141,10 +165,10 @@ def build(force=False):
         text = open(os.path.join(CSRC, name)).read()
         cpp = os.path.join(OUT, name.replace(".hip", "_hostsim.cpp"))
         with open(cpp, "w") as f:
-            f.write(rewrite_lockstep(rewrite_asm(rewrite_dynamic_lds(rewrite_launches(text)))))
+            f.write(rewrite_declared_accesses(rewrite_lockstep(rewrite_asm(rewrite_dynamic_lds(rewrite_launches(text))))))
         objects.append(cpp)
     cmd = [CLANG, "-std=c++17", "-O2", "-g", "-fPIC", "-shared", "-D__HIP__", "-Wno-everything", "-I", HERE, "-I", OUT, "-I", CSRC,
-           "-I", os.path.join(ROOT, "include"), "-o", LIB, os.path.join(HERE, "hostsim.cpp")] + objects
+           "-I", os.path.join(ROOT, "include"), "-o", LIB, os.path.join(HERE, "hostsim.cpp"), os.path.join(HERE, "order.cpp")] + objects
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError("host simulation build failed:\n" + proc.stderr[-6000:])

@@ -50,27 +50,47 @@ typedef int hipError_t;
 enum { hipSuccess = 0, hipErrorInvalidValue = 1 };
 enum { hipFuncAttributeMaxDynamicSharedMemorySize = 8, hipDeviceAttributeMultiprocessorCount = 63 };
 inline hipError_t hipGetLastError() { return hipSuccess; }
-inline const char* hipGetErrorString(hipError_t) { return "host simulation"; }
+inline const char* hipGetErrorString(hipError_t e) { return e == 2 ? "stream order violation (host simulation)" : "host simulation"; }
 inline hipError_t hipGetDevice(int* d) { *d = 0; return hipSuccess; }
 inline hipError_t hipDeviceGetAttribute(int* v, int, int) { *v = 256; return hipSuccess; }
 template <typename F> inline hipError_t hipFuncSetAttribute(F, int, int) { return hipSuccess; }
 template <typename T> inline hipError_t hipGetSymbolAddress(void** out, T* sym) { *out = (void*)sym; return hipSuccess; }
 
 // Copies, events and pinned memory for the streaming code: everything completes at the call (one of the
-// orders the streams allow), so events and waits have nothing left to do.
+// orders the streams allow).  What events and waits still do is bookkeeping: every stream carries a vector
+// clock (order.cpp), copies declare the bytes they read and write, and a copy that is not ordered after an
+// earlier overlapping access on another stream fails like a failed HIP call.
+extern "C" {
+uint64_t hostsim_order_snapshot(uint64_t stream);
+void hostsim_order_wait(uint64_t stream, uint64_t handle);
+int hostsim_order_enqueue(uint64_t stream, const char* what, int n, const uint64_t* lo, const uint64_t* bytes, const int* is_write);
+}
+enum { hipErrorStreamOrder = 2 };
+struct hostsim_event { uint64_t snapshot; };
 typedef struct hostsim_event* hipEvent_t;
 enum hipMemcpyKind { hipMemcpyHostToDevice = 1, hipMemcpyDeviceToHost = 2, hipMemcpyDeviceToDevice = 3 };
 enum { hipEventDisableTiming = 2, hipHostMallocDefault = 0 };
-inline hipError_t hipMemcpyAsync(void* dst, const void* src, size_t n, hipMemcpyKind, hipStream_t) { memcpy(dst, src, n); return hipSuccess; }
-inline hipError_t hipMemcpy2DAsync(void* dst, size_t dpitch, const void* src, size_t spitch, size_t width, size_t height, hipMemcpyKind,
-                                   hipStream_t) {
-    for (size_t r = 0; r < height; ++r) memcpy((char*)dst + r * dpitch, (const char*)src + r * spitch, width);
-    return hipSuccess;
+inline hipError_t hostsim_declare(hipStream_t stream, const char* what, const void* read, size_t read_bytes, void* write, size_t write_bytes) {
+    const uint64_t lo[2] = {(uint64_t)(uintptr_t)read, (uint64_t)(uintptr_t)write}, bytes[2] = {read_bytes, write_bytes};
+    const int is_write[2] = {0, 1};
+    return hostsim_order_enqueue((uint64_t)(uintptr_t)stream, what, 2, lo, bytes, is_write) ? hipErrorStreamOrder : hipSuccess;
 }
-inline hipError_t hipEventCreateWithFlags(hipEvent_t* e, unsigned) { *e = reinterpret_cast<hipEvent_t>(malloc(1)); return hipSuccess; }
-inline hipError_t hipEventDestroy(hipEvent_t e) { free(e); return hipSuccess; }
-inline hipError_t hipEventRecord(hipEvent_t, hipStream_t) { return hipSuccess; }
-inline hipError_t hipStreamWaitEvent(hipStream_t, hipEvent_t, unsigned) { return hipSuccess; }
+inline hipError_t hipMemcpyAsync(void* dst, const void* src, size_t n, hipMemcpyKind, hipStream_t stream) {
+    const hipError_t e = hostsim_declare(stream, "copy", src, n, dst, n);
+    memcpy(dst, src, n);
+    return e;
+}
+inline hipError_t hipMemcpy2DAsync(void* dst, size_t dpitch, const void* src, size_t spitch, size_t width, size_t height, hipMemcpyKind,
+                                   hipStream_t stream) {
+    const hipError_t e = height ? hostsim_declare(stream, "2-D copy", src, (height - 1) * spitch + width, dst, (height - 1) * dpitch + width)
+                                : hipSuccess;
+    for (size_t r = 0; r < height; ++r) memcpy((char*)dst + r * dpitch, (const char*)src + r * spitch, width);
+    return e;
+}
+inline hipError_t hipEventCreateWithFlags(hipEvent_t* e, unsigned) { *e = new hostsim_event{0}; return hipSuccess; }
+inline hipError_t hipEventDestroy(hipEvent_t e) { delete e; return hipSuccess; }
+inline hipError_t hipEventRecord(hipEvent_t e, hipStream_t s) { e->snapshot = hostsim_order_snapshot((uint64_t)(uintptr_t)s); return hipSuccess; }
+inline hipError_t hipStreamWaitEvent(hipStream_t s, hipEvent_t e, unsigned) { hostsim_order_wait((uint64_t)(uintptr_t)s, e->snapshot); return hipSuccess; }
 inline hipError_t hipHostMalloc(void** p, size_t n, unsigned) { *p = malloc(n); return *p ? hipSuccess : hipErrorInvalidValue; }
 inline hipError_t hipHostFree(void* p) { free(p); return hipSuccess; }
 

@@ -12,9 +12,10 @@ import os
 
 import torch
 
-from .order import CLOCKS, OrderedLibrary
+from . import order
 
 ACTIVE = os.environ.get("FLEXTRAIN_HOSTSIM") == "1"
+CLOCKS = None        # order.Clocks of the simulated library, set by activate()
 
 
 def _current():
@@ -56,10 +57,10 @@ class _Stream:
         self.cuda_stream = 0x1000 * _Stream._handles       # a distinct non-null handle per stream object
 
     def synchronize(self):
-        CLOCKS.host_sync(CLOCKS.snapshot(self.cuda_stream))
+        CLOCKS.stream_sync(self.cuda_stream)
 
     def wait_stream(self, other):
-        CLOCKS.wait(self.cuda_stream, CLOCKS.snapshot(other.cuda_stream))
+        CLOCKS.wait_stream(self.cuda_stream, other.cuda_stream)
 
     def wait_event(self, event):
         event.wait(self)
@@ -110,7 +111,9 @@ def activate():
 
     from . import sim
 
-    _lib._lib = OrderedLibrary(sim.lib())
+    global CLOCKS
+    _lib._lib = sim.lib()
+    CLOCKS = order.Clocks(sim.lib())
     default = _Stream()
     default.cuda_stream = 0
     current = [default]

@@ -80,44 +80,50 @@ def test_tensors_of_the_simulated_gpu_suite_end_at_a_guard_page():
 
 
 def test_a_removed_wait_in_the_streamed_optimizer_step_is_reported():
-    """The happens-before check of the simulated run: the pipelined optimizer step over the layer rings passes
-    with many cross-stream pairs examined, and taking away any one class of its waits (the compute stream's
-    wait for a layer's fetches, the outbound stream's wait for the update, the inbound stream's wait before a
-    slot is refilled) raises StreamOrderError at the enqueue that is no longer ordered."""
+    """The happens-before check of the simulated run: the pipelined optimizer step over the layer rings and the
+    library's own streamed chunk pass with many cross-stream pairs examined, and with the waits of any one of
+    the three streams taken away the enqueue that is no longer ordered fails and says why."""
     prologue = """
         import os, sys
         os.environ["FLEXTRAIN_HOSTSIM"] = "1"
         sys.path.insert(0, "tests")
         import torch
-        from hostsim import mode, order
+        from hostsim import mode
         mode.ACTIVE = True
         mode.activate()
         import test_gpu_layer_ring as t
         from flextrain_amd.layer_ring import ring_optimizer_step
+        from flextrain_amd.optim import flextrain_adamw_step_streamed
         from flextrain_amd.streams import EventBook, StreamBundle
         dev = torch.device("cpu")
-        def run():
+        streams = StreamBundle.create(dev)
+        def rings():
             specs, buf = t._make(dev, 5, 2, 2, 7)
-            streams = StreamBundle.create(dev)
-            return streams, ring_optimizer_step(buf, streams, EventBook(), n_gpu_opt_layers=2, step_num=4, **t.HP)
+            return ring_optimizer_step(buf, streams, EventBook(), n_gpu_opt_layers=2, step_num=4, **t.HP)
+        def chunk():
+            from flextrain_amd.host_memory import LocalPinnedHostBackend
+            n, be = 40000, LocalPinnedHostBackend()
+            p, m, v = (be.allocate_tensor((n,), torch.float32) for _ in range(3))
+            g = be.allocate_tensor((n,), torch.bfloat16)
+            return flextrain_adamw_step_streamed(p, g, m, v, streams=streams, sub_elems=4096, n_slots=2, step=1, **t.HP)
+        def deafen(role):
+            mode.CLOCKS.deafen(getattr(streams, role).cuda_stream)
     """
     ok = _child(prologue + """
-        assert run()[1] == 0
-        assert order.CLOCKS.checked > 50, order.CLOCKS.checked
-        print("fine", order.CLOCKS.checked)
+        assert rings() == 0 and chunk() == 0
+        assert mode.CLOCKS.checked > 50 and mode.CLOCKS.last_violation == "", (mode.CLOCKS.checked, mode.CLOCKS.last_violation)
+        print("fine", mode.CLOCKS.checked)
     """)
     assert ok.returncode == 0 and "fine" in ok.stdout, ok.stderr[-2000:]
     for role in ("compute", "outbound", "inbound"):
         bad = _child(prologue + f"""
-        streams = StreamBundle.create(dev)
-        deaf = streams.{role}.cuda_stream
-        plain = order.CLOCKS.wait
-        order.CLOCKS.wait = lambda sid, clock: None if sid == deaf else plain(sid, clock)   # this stream waits for nothing
-        StreamBundle.create = classmethod(lambda cls, *a, **k: streams)
-        try:
-            run()
-            print("unnoticed")
-        except order.StreamOrderError as exc:
-            print("reported:", exc)
+        deafen("{role}")
+        for schedule in (rings, chunk):
+            try:
+                print(schedule.__name__, "returned", schedule())
+            except RuntimeError as exc:
+                print(schedule.__name__, "raised", exc)
+            print("violation:", mode.CLOCKS.last_violation)
         """)
-        assert bad.returncode == 0 and "reported:" in bad.stdout and "unnoticed" not in bad.stdout, (role, bad.stdout[-500:], bad.stderr[-1500:])
+        out = bad.stdout
+        assert bad.returncode == 0 and out.count("is not ordered after") == 2 and "returned 0" not in out, (role, out[-900:], bad.stderr[-1500:])
