@@ -167,11 +167,26 @@ def build(force=False):
         with open(cpp, "w") as f:
             f.write(rewrite_declared_accesses(rewrite_lockstep(rewrite_asm(rewrite_dynamic_lds(rewrite_launches(text))))))
         objects.append(cpp)
-    cmd = [CLANG, "-std=c++17", "-O2", "-g", "-fPIC", "-shared", "-D__HIP__", "-Wno-everything", "-I", HERE, "-I", OUT, "-I", CSRC,
-           "-I", os.path.join(ROOT, "include"), "-o", LIB, os.path.join(HERE, "hostsim.cpp"), os.path.join(HERE, "order.cpp")] + objects
-    proc = subprocess.run(cmd, capture_output=True, text=True)
+    flags = [CLANG, "-std=c++17", "-O2", "-g", "-fPIC", "-D__HIP__", "-Wno-everything", "-I", HERE, "-I", OUT, "-I", CSRC,
+             "-I", os.path.join(ROOT, "include")]
+    units = [os.path.join(HERE, "hostsim.cpp"), os.path.join(HERE, "order.cpp")] + objects
+
+    def compile_one(src):
+        obj = os.path.join(OUT, os.path.basename(src) + ".o")
+        proc = subprocess.run(flags + ["-c", src, "-o", obj], capture_output=True, text=True)
+        if proc.returncode != 0:
+            raise RuntimeError(f"host simulation build failed ({os.path.basename(src)}):\n" + proc.stderr[-6000:])
+        return obj
+
+    from concurrent.futures import ThreadPoolExecutor
+
+    with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as pool:      # one compiler process per source
+        objs = list(pool.map(compile_one, units))
+    # linked under a temporary name and renamed: a process that has the old library mapped keeps it
+    proc = subprocess.run([CLANG, "-shared", "-o", LIB + ".tmp"] + objs, capture_output=True, text=True)
     if proc.returncode != 0:
-        raise RuntimeError("host simulation build failed:\n" + proc.stderr[-6000:])
+        raise RuntimeError("host simulation link failed:\n" + proc.stderr[-6000:])
+    os.replace(LIB + ".tmp", LIB)
     return LIB
 
 

@@ -41,6 +41,10 @@ def test_streamed_adamw_chunk(n, sub, slots, ring, staged_copy):
         assert L.fx_adamw_stream_chunk(P(hp_), P(hg), P(hm), P(hv), P(hc), 0 if staged_copy else 1, n, 0, 2, 0, hp["lr"], hp["beta1"],
                                        hp["beta2"], hp["eps"], hp["weight_decay"], 1 - hp["beta1"] ** step, 1 - hp["beta2"] ** step,
                                        P(ws), ws_bytes, sub, slots, S, S + 1, S + 2, handle if ring else None) == 0
+        # as a caller does before it reads the results (and before the next call reads them as its inputs): the
+        # host waits for the copies out, and for the kernels where they write the bf16 copy themselves
+        L.hostsim_order_stream_sync(ctypes.c_uint64(S + 2))
+        L.hostsim_order_stream_sync(ctypes.c_uint64(S + 1))
         p, m, v, c = o_adam.adamw_step(p, gr, m, v, step=step, **hp)
         torch.testing.assert_close(hp_, p, rtol=1e-5, atol=1e-7)
         torch.testing.assert_close(hm, m, rtol=1e-5, atol=1e-9)
