@@ -1122,17 +1122,25 @@ def main():
         op_rows += run_extra(torch, ops, dev, stream, rn, [t.strip() for t in args.only.split(",") if t.strip()])
         if not any("error" in r for r in op_rows):
             _progress("mfma probe")
-            mfma_probe = run_mfma_probe(torch, dev, stream)
+            try:
+                mfma_probe = run_mfma_probe(torch, dev, stream)
+            except Exception as exc:  # noqa: BLE001 - the probe is an annotation: its failure must not cost the rows
+                _progress(f"mfma probe FAILED: {type(exc).__name__}: {exc}")
+                op_rows.append({"op": "mfma_probe.FAILED", "unit": "", "error": f"{type(exc).__name__}: {exc}"})
+            sustained = (mfma_probe or {}).get("random_operands", {}).get("tflops", 0.0)
             for row in op_rows:
-                if row["unit"] == "TFLOP/s":
-                    row["frac_of_sustained_mfma_random_operands"] = round(
-                        row["achieved"] / mfma_probe["random_operands"]["tflops"], 4)
+                if row["unit"] == "TFLOP/s" and sustained > 0:
+                    row["frac_of_sustained_mfma_random_operands"] = round(row["achieved"] / sustained, 4)
     _progress("cpu baselines")
 
     # -------------------------------------------------------- CPU baseline
     cpu = None
     if not args.no_cpu and not args.no_extra:
-        op_rows += run_cpu_baselines(torch, [t.strip() for t in args.only.split(",") if t.strip()])
+        try:
+            op_rows += run_cpu_baselines(torch, [t.strip() for t in args.only.split(",") if t.strip()])
+        except Exception as exc:  # noqa: BLE001 - reported in the line; the measured GPU rows are kept
+            _progress(f"cpu baselines FAILED: {type(exc).__name__}: {exc}")
+            op_rows.append({"op": "cpu_baselines.FAILED", "unit": "", "error": f"{type(exc).__name__}: {exc}"})
     if not args.no_cpu:
         from oracle import glu as o_glu
         from oracle import rope as o_rope

@@ -137,6 +137,8 @@ def activate():
     torch.cuda.Event = _Event
     torch.cuda.memory_allocated = lambda device=None: 0
     torch.cuda.set_device = lambda device: None
+    torch.cuda.set_stream = lambda s: current.__setitem__(len(current) - 1, s)
+    torch.cuda.empty_cache = lambda: None
     torch.cuda.init = lambda: None
     # a tensor "moved to the GPU" is a copy there, and the tests rely on it (in-place kernels must not touch
     # the host original that the oracle is given afterwards); on one device Tensor.to returns the tensor itself
@@ -144,9 +146,18 @@ def activate():
 
     plain_clone = torch.Tensor.clone
 
+    def simulated(d):
+        """A CUDA device named by the caller is the simulated one: host memory."""
+        if isinstance(d, (torch.device, str)) and not isinstance(d, torch.dtype) and torch.device(d).type == "cuda":
+            return torch.device("cpu")
+        return d
+
     def to(self, *args, **kwargs):
-        out = plain_to(self, *args, **kwargs)
         moved = "device" in kwargs or any(isinstance(a, (torch.device, str)) for a in args)
+        args = tuple(simulated(a) for a in args)
+        if "device" in kwargs:
+            kwargs["device"] = simulated(kwargs["device"])
+        out = plain_to(self, *args, **kwargs)
         if not moved:
             return out
         return _behind_a_guard_page(plain_clone(out) if out is self else out)

@@ -56,3 +56,18 @@ def test_a_failing_leg_is_reported_and_ends_the_gpu_legs(monkeypatch):
 def test_more_than_one_gpu_is_refused():
     proc = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert proc.returncode == 2 and "one GPU only" in proc.stderr and proc.stdout == ""
+
+
+def test_the_headline_path_runs_through_to_the_json_line():
+    """bench.py itself, unchanged and at its real shapes, on a library whose launches return at once
+    (tests/hostsim/bench_dry_run.py): the headline workload, one leg and the assembly of the final line
+    raise no Python error.  The whole script takes five minutes that way and is run by hand."""
+    from tests.hostsim.build import CLANG
+
+    if not os.path.exists(CLANG):
+        import pytest
+
+        pytest.skip("the host simulation is compiled with " + CLANG)
+    proc = subprocess.run([sys.executable, "-m", "tests.hostsim.bench_dry_run", "--only", "disp"], cwd=ROOT, capture_output=True,
+                          text=True, timeout=900)
+    assert proc.returncode == 0 and "failed legs: none" in proc.stdout, (proc.stdout[-500:], proc.stderr[-2000:])
