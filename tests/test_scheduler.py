@@ -205,3 +205,33 @@ def test_a_huge_window_costs_nothing():
     _, val, choices = _product(c, buf_size=(1 << 31) - 1)
     oval, ochoices = o_dp.solve_scheduler(c["compute"], c["durations"], c["sizes"], c["deadline"], c["time_scale"], c["N"])
     assert val == oval == 35700.0 and choices == ochoices.tolist()
+
+
+@pytest.mark.skipif(not os.path.exists(REF), reason="compiled reference solver (oracle/_ref) not built")
+def test_edge_problems_against_compiled_reference():
+    """Windows of 1 to 4096 ticks (most far narrower than the band), 1 / 10 / 100 ticks per ms, zero compute
+    times and durations, deadlines that cut the schedule short, integer values (ties): value and option
+    vector as the compiled reference gives them, and untouched choices where it finds no schedule."""
+    ref = ctypes.CDLL(REF)
+    ref.solve_scheduler.argtypes = [ctypes.c_int] * 3 + [ctypes.c_void_p] * 3 + [ctypes.c_double, ctypes.c_int, ctypes.c_int,
+                                                                                 ctypes.c_void_p]
+    ref.solve_scheduler.restype = ctypes.c_double
+    rng = np.random.default_rng(5)
+    feasible = 0
+    for trial in range(1500):
+        T, k, N = int(rng.integers(1, 40)), int(rng.integers(1, 5)), int(rng.integers(1, 12))
+        scale = int(rng.choice([1, 10, 100]))
+        compute = rng.uniform(0.0, 12.0, T)
+        durations = rng.uniform(0.0, 30.0, (T, k))
+        sizes = rng.integers(1, 6, (T, k)).astype(np.float64) if trial % 2 else rng.uniform(0.5, 50, (T, k))
+        deadline = float(compute.sum() + (durations.max(axis=1).sum() + 1000.0 if trial % 3 else rng.uniform(0, 20)))
+        buf = int(rng.choice([1, 2, 3, 7, 64, 300, 2048, 4096]))
+        c = dict(compute=compute, durations=durations, sizes=sizes, deadline=deadline, time_scale=scale, N=N, buf_size=buf)
+        _, val, choices = _product(c)
+        rchoices = np.full(T, -1, dtype=np.int32)
+        rval = ref.solve_scheduler(T, N, k, compute.ctypes.data, durations.ctypes.data, sizes.ctypes.data, deadline, scale, buf,
+                                   rchoices.ctypes.data)
+        assert val == rval, trial
+        assert choices == rchoices.tolist(), trial
+        feasible += val != 0.0
+    assert feasible > 50
